@@ -556,6 +556,69 @@ int vlm_vit_set_block(void* handle, int i, const vlm_vit_block* w);
 int vlm_vit_set_globals(void* handle, const vlm_vit_globals* g);
 int vlm_vit_forward(void* handle, const vlm_vit_args* a, void* stream);
 
+/* ------------------------------------------------------------------------------------------------------------------
+ * Operators of decoders with an fp32 residual stream, matrix-state recurrences, latent attention and mixtures of experts
+ * (models/garesun).  "T" pointers are bf16 (dtype 0) or fp32 (dtype 1): dtype 1 is the true 32-bit serving mode.  Norm
+ * statistics, scores, softmax weights, gates, routers, recurrent state and the residual sum are fp32 in both.
+ * ------------------------------------------------------------------------------------------------------------------ */
+
+/* C[b][m][n] (+)= sum_k A[b][m][k] W[b][n][k]: any shape / leading dimension, each operand bf16 or fp32, fp32 FMAs in a fixed
+ * order per row (csrc/linear_any.hip).  accumulate needs an fp32 C. */
+int vlm_linear_any(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc, int a_f32, int w_f32,
+                   int c_f32, int batch, long strideA, long strideW, long strideC, int accumulate, void* stream);
+
+/* csrc/stream_f32.hip: x is the fp32 stream [rows][D] */
+int vlm_embed_scale_f32(const void* ids, const void* table, float scale, void* x, int rows, int D, int vocab, int dtype, void* stream);
+int vlm_layernorm_nobias(const void* x, const void* w, void* out, int rows, int D, long ldo, float eps, int dtype, void* stream);
+int vlm_stream_add(void* x, const void* a, long lda, const void* b, long ldb, int rows, int D, int dtype, void* stream);
+int vlm_unit_rms_add(void* x, const void* y, long ldy, const void* w, int rows, int D, float eps, int dtype, void* stream);
+int vlm_gelu_tanh_gate_rows(const void* g, long ldg, const void* table, long ldt, const void* ids, int col0, void* out, long ldo,
+                            int rows, int dim, int vocab, int dtype, void* stream);
+
+/* csrc/linear_recurrence.hip: S_t = a_t S_(t-1) + b_t k_t v_t^T, o_t = S_t^T q_t per head, state fp32 per sequence slot.
+ * gated = 0: a = decay[h], b = 1, rotate-half positions on the first rot_dims dimensions of q and k (inv_freq fp32
+ * [rot_dims / 2]); gated = 1: exponential gates with a running maximum, normaliser column, denominator (see the file).
+ * Then per head: unit RMS (eps), times normw (T [H * Dv], may be NULL), times silu (gate_act 0) or sigmoid (1) of g. */
+typedef struct vlm_recurrence_args {
+  const void *q, *k, *v, *g;            /* T: row t at + t * ld, head h at + h * D (q, k) / + h * Dv (v, g) */
+  long ldq, ldk, ldv, ldg;
+  const void *ipre, *fpre;              /* gated: T pre-activations [.][H] at ldi / ldf, biases T [H] */
+  long ldi, ldf;
+  const void *ib, *fb;
+  float cap;
+  const float* decay;                   /* not gated: fp32 [H] */
+  const float* inv_freq;
+  int rot_dims;
+  float qscale, kscale;                 /* applied after the rotation */
+  const void* normw;
+  int gate_act;
+  float eps;
+  const int *seg_start, *seg_slot, *seg_pos0; /* [nseg + 1] token ranges, [nseg] state slots, [nseg] position of the first token */
+  float* state;                         /* [slots][H][D][Dv + gated] */
+  float* mstate;                        /* gated: [slots][H] running maximum */
+  float* mtok;                          /* gated scratch: [ntok][H] */
+  float* mprev;                         /* gated scratch: [nseg][H] */
+  float* raw;                           /* scratch fp32 [ntok][H][Dv + gated] */
+  void* out;                            /* T [ntok] rows at ldo */
+  long ldo;
+  int H, D, Dv, gated;
+} vlm_recurrence_args;
+int vlm_linear_recurrence(const vlm_recurrence_args* a, int nseg, int ntok, int dtype, void* stream);
+
+/* csrc/latent_attn.hip: pool T [pages][64][R + Dr]; token t belongs to block-table row tok_seq[t] at position tok_pos[t] */
+int vlm_latent_kv_write(const void* d, long ldd, const void* w, int R, int Dr, const void* inv_freq, const void* tok_seq,
+                        const void* tok_pos, const void* block_table, int max_pages, void* pool, float eps, int rows, int dtype,
+                        void* stream);
+int vlm_rope_pairs_rows(const void* q, long ldq, long head_stride, int H, int Dr, const void* inv_freq, const void* tok_pos, void* out,
+                        long ldo, long out_head_stride, int rows, int dtype, void* stream);
+int vlm_latent_attn(const void* q, const void* pool, const void* tok_seq, const void* tok_pos, const void* block_table, int max_pages,
+                    int H, int R, int Dr, float scale, const void* gate, long ldgate, void* out, int rows, int dtype, void* stream);
+
+/* csrc/moe.hip */
+int vlm_moe_route(const void* logits, int T, int E, int top, void* gate, void* idx, void* wgt, void* stream);
+int vlm_moe_relu2_gate(const void* up, long ldu, const void* gate, int E, int ff, int shared, void* out, long ldo, int rows, int dtype,
+                       void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -92,6 +92,17 @@ class VitArgs(C.Structure):
                 ("uniform_segments", c_int)]
 
 
+class RecurrenceArgs(C.Structure):
+    """vlm_recurrence_args (include/vlm_hip.h): one matrix-state recurrence layer over the segments of a step"""
+    _fields_ = ([(n, c_void_p) for n in ("q", "k", "v", "g")] + [(n, C.c_long) for n in ("ldq", "ldk", "ldv", "ldg")]
+                + [("ipre", c_void_p), ("fpre", c_void_p), ("ldi", C.c_long), ("ldf", C.c_long), ("ib", c_void_p), ("fb", c_void_p),
+                   ("cap", c_float), ("decay", c_void_p), ("inv_freq", c_void_p), ("rot_dims", c_int), ("qscale", c_float),
+                   ("kscale", c_float), ("normw", c_void_p), ("gate_act", c_int), ("eps", c_float), ("seg_start", c_void_p),
+                   ("seg_slot", c_void_p), ("seg_pos0", c_void_p), ("state", c_void_p), ("mstate", c_void_p), ("mtok", c_void_p),
+                   ("mprev", c_void_p), ("raw", c_void_p), ("out", c_void_p), ("ldo", C.c_long), ("H", c_int), ("D", c_int),
+                   ("Dv", c_int), ("gated", c_int)])
+
+
 DECODE_FUSED_TAIL = 1                       # vlm_decode_args.flags
 DECODE_ACT16 = 2                            # `act` holds 16 x intermediate_size elements (tiled hand-over to the down projection)
 TUNE_MFMA_GEMV, TUNE_ATTN_PAGESPLIT, TUNE_GEMV_VARIANT, TUNE_ATTN_MERGE = 6, 7, 8, 9  # vlm_llm_set_tuning keys (include/vlm_hip.h)
@@ -173,6 +184,21 @@ SIGNATURES = {
     "vlm_vit_set_block": (c_int, [c_void_p, c_int, P(VitBlock)]),
     "vlm_vit_set_globals": (c_int, [c_void_p, P(VitGlobals)]),
     "vlm_vit_forward": (c_int, [c_void_p, P(VitArgs), c_void_p]),
+    "vlm_linear_any": (c_int, [c_void_p] * 3 + [c_int] * 3 + [C.c_long] * 3 + [c_int] * 4 + [C.c_long] * 3 + [c_int, c_void_p]),
+    "vlm_embed_scale_f32": (c_int, [c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
+    "vlm_layernorm_nobias": (c_int, [c_void_p] * 3 + [c_int, c_int, C.c_long, c_float, c_int, c_void_p]),
+    "vlm_stream_add": (c_int, [c_void_p, c_void_p, C.c_long, c_void_p, C.c_long, c_int, c_int, c_int, c_void_p]),
+    "vlm_unit_rms_add": (c_int, [c_void_p, c_void_p, C.c_long, c_void_p, c_int, c_int, c_float, c_int, c_void_p]),
+    "vlm_gelu_tanh_gate_rows": (c_int, [c_void_p, C.c_long, c_void_p, C.c_long, c_void_p, c_int, c_void_p, C.c_long, c_int, c_int,
+                                        c_int, c_int, c_void_p]),
+    "vlm_linear_recurrence": (c_int, [P(RecurrenceArgs), c_int, c_int, c_int, c_void_p]),
+    "vlm_latent_kv_write": (c_int, [c_void_p, C.c_long, c_void_p, c_int, c_int] + [c_void_p] * 4 + [c_int, c_void_p, c_float, c_int,
+                                    c_int, c_void_p]),
+    "vlm_rope_pairs_rows": (c_int, [c_void_p, C.c_long, C.c_long, c_int, c_int, c_void_p, c_void_p, c_void_p, C.c_long, C.c_long,
+                                    c_int, c_int, c_void_p]),
+    "vlm_latent_attn": (c_int, [c_void_p] * 5 + [c_int] * 4 + [c_float, c_void_p, C.c_long, c_void_p, c_int, c_int, c_void_p]),
+    "vlm_moe_route": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "vlm_moe_relu2_gate": (c_int, [c_void_p, C.c_long, c_void_p, c_int, c_int, c_int, c_void_p, C.c_long, c_int, c_int, c_void_p]),
 }
 
 _lib = None

@@ -308,6 +308,7 @@ class BatchGenerator:
 
     def _decode_rows(self, width: int):
         """One decode step over rows 0..width-1 of the state: tok <- sampled token, pos and ctx advanced by one."""
+        self._st.row_seqs = [row.seq for row in self._rows]     # (engines that address state by sequence slot, not by table row)
         if self._py_sampler is not None or any(row.py_procs for row in self._rows):
             return self._decode_rows_eager(width)
         self.lm.decode_step_rows(self._st, width, self._table, self._sargs, use_graph=self.use_graph,
@@ -372,7 +373,8 @@ class BatchGenerator:
             if st.B == cap and not getattr(st, "in_use", False):
                 break
         else:
-            st = DecodeState(lm, cap)
+            # a language model with its own step function brings its own row state (same fields: tok / pos / ctx / step / ...)
+            st = lm.new_decode_state(cap) if hasattr(lm, "new_decode_state") else DecodeState(lm, cap)
             parked.append(st)
         st.in_use = True
         for buf in (st.tok, st.pos, st.ctx, st.step):
@@ -746,3 +748,41 @@ def generate_batch_continuous(model, input_ids_list, pixel_values_list, grids, *
     gen.close()
     stats.wall_time = total
     return [results[u] for u in uids], stats
+
+
+class TraceSession:
+    """Replay of an externally scheduled trace on the model's ragged step function: the caller says which requests bring
+    which tokens in each step (prompt portions and decoded tokens mixed) and which logits it wants; this class owns the
+    bookkeeping the generators do for themselves - a cache per live request from the model's pool (`make_cache`), release of
+    pages and state slot when a request ends, so both are used again by later requests.  Nothing is sampled."""
+
+    def __init__(self, model):
+        self.model = model
+        self.lm = model.language_model
+        if not hasattr(self.lm, "step"):
+            raise NotImplementedError(f"{type(self.lm).__name__} has no ragged step function")
+        self._live: Dict[Any, list] = {}
+
+    def step(self, entries, end=()):
+        """entries: [(request id, next token ids, wanted indices)] -> fp32 logits on the host [n wanted, vocab] or None"""
+        batch, want = [], []
+        for rid, tokens, w in entries:
+            cache = self._live.get(rid)
+            if cache is None:
+                cache = self._live[rid] = self.lm.make_cache()
+            batch.append((cache[0]._seq, np.asarray(tokens, dtype=np.int32)))
+            want.append(list(w))
+        logits = self.lm.step(batch, want=want) if batch else None
+        out = logits.float().cpu() if logits is not None else None      # (the copy also orders the release below behind the step)
+        for rid in end:
+            cache = self._live.pop(rid, None)
+            if cache is not None:
+                if out is None:
+                    torch.cuda.current_stream().synchronize()
+                cache[0]._seq.release()
+        return out
+
+    def close(self):
+        for cache in self._live.values():
+            cache[0]._seq.release()
+        self._live.clear()

@@ -26,7 +26,9 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # D = 80 kernel needs 218 registers instead of 172 + 80, D = 128 fits two waves per SIMD (212 vs 292), and the 128-tile
 # GEMM loses its 5472 accumulator moves.  Results are bit-identical (profiles/r02_attn_prefill_probe.txt).
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
-         "-Wno-unused-variable", "-Wno-pass-failed", "-mllvm", "-amdgpu-mfma-vgpr-form"]
+         "-Wno-unused-variable", "-Wno-pass-failed", "-mllvm", "-amdgpu-mfma-vgpr-form",
+         # no packed fp32 VALU forms (v_pk_add / mul / fma_f32): the compiler may not form them from scalar or float2 code
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 # measurement builds only (e.g. VLM_BUILD_DEFINES="VLM_GEMM_ABLATION GEMM_STAMPS"): never set for the shipped library
 FLAGS += ["-D" + d for d in os.environ.get("VLM_BUILD_DEFINES", "").split()]
 

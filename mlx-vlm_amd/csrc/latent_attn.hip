@@ -1,0 +1,215 @@
+// Latent attention: every head reads ONE cached row per token - a low-rank latent c [R] (RMS-normed with a weight) and one
+// rotated key part kr [Dr] shared by all heads.  Per-head keys and values are linear maps of c (k_h = U_k,h c, v_h = U_v,h c),
+// so the maps are moved to the query and output side ("absorbed"): with q'_h = U_k,h^T q_h the score of key j is
+//
+//     s_hj = scale * (q'_h . c_j + rope(q_rot,h) . kr_j)          o_h = U_v,h sum_j softmax(s_h)_j c_j
+//
+// and attention runs straight over the cached rows [c | kr] with "head dim" R + Dr for scores and R for values; nothing
+// per head is ever cached or materialised per key.  A layer may read ANOTHER layer's cache (same R, Dr, rotation).
+//
+//   vlm_latent_kv_write      d = W_dkv h rows -> c = d[:R] * rsqrt(mean(d[:R]^2) + eps) * w, kr = rope_pairs(d[R:], pos) into the
+//                            paged pool [page][64][R + Dr] (T-typed) of the token's sequence
+//   vlm_rope_pairs_rows      rotate the Dr-wide rotary part of every head's query (pairs (2 i, 2 i + 1)) into the fp32 query
+//                            buffer behind the absorbed part
+//   vlm_latent_attn          causal softmax attention of fp32 queries [T][H][R + Dr] over the pool; key tiles start at
+//                            multiples of 256 counted from the sequence's first token, so the arithmetic of a token does not
+//                            depend on how its prompt was cut; output fp32 [T][H][R], times sigmoid(gate[t][h]) when a gate
+//                            is given
+// Scores, softmax and the weighted sum are fp32.  dtype: 0 = bf16, 1 = fp32 for the T-typed pointers.
+#include "common.hpp"
+#include "../../include/vlm_hip.h"
+
+namespace {
+
+template <typename T> __device__ __forceinline__ float ld_f(const T* p);
+template <> __device__ __forceinline__ float ld_f<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float ld_f<bf16_t>(const bf16_t* p) { return bf2f(*p); }
+template <typename T> __device__ __forceinline__ void st_f(T* p, float v);
+template <> __device__ __forceinline__ void st_f<float>(float* p, float v) { *p = v; }
+template <> __device__ __forceinline__ void st_f<bf16_t>(bf16_t* p, float v) { *p = f2bf(v); }
+
+constexpr int PAGE = 64;
+
+template <typename T>
+__global__ __launch_bounds__(256) void latent_kv_write_kernel(const T* __restrict__ d, long ldd, const T* __restrict__ w, int R, int Dr,
+                                                              const float* __restrict__ inv_freq, const int* __restrict__ tok_seq,
+                                                              const int* __restrict__ tok_pos, const int* __restrict__ block_table,
+                                                              int max_pages, T* __restrict__ pool, float eps) {
+  __shared__ float red[4];
+  const long t = blockIdx.x;
+  const T* row = d + t * ldd;
+  const int pos = tok_pos[t];
+  const int page = block_table[(long)tok_seq[t] * max_pages + pos / PAGE];
+  T* dst = pool + ((long)page * PAGE + pos % PAGE) * (R + Dr);
+  float q = 0.f;
+  for (int i = threadIdx.x; i < R; i += 256) {
+    const float v = ld_f(row + i);
+    q += v * v;
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) q += __shfl_xor(q, o);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = q;
+  __syncthreads();
+  const float r = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)R + eps);
+  for (int i = threadIdx.x; i < R; i += 256) st_f(dst + i, ld_f(row + i) * r * ld_f(w + i));
+  for (int i = threadIdx.x; i < Dr / 2; i += 256) {
+    const float u = ld_f(row + R + 2 * i), v = ld_f(row + R + 2 * i + 1);
+    float sn, cs;
+    sincosf((float)pos * inv_freq[i], &sn, &cs);
+    st_f(dst + R + 2 * i, u * cs - v * sn);
+    st_f(dst + R + 2 * i + 1, v * cs + u * sn);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void rope_pairs_rows_kernel(const T* __restrict__ q, long ldq, long head_stride, int H, int Dr,
+                                                              const float* __restrict__ inv_freq, const int* __restrict__ tok_pos,
+                                                              float* __restrict__ out, long ldo, long out_head_stride, int rows) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  const int hp = Dr / 2;
+  if (i >= (long)rows * H * hp) return;
+  const int pi = (int)(i % hp), h = (int)((i / hp) % H);
+  const long t = i / ((long)hp * H);
+  const T* src = q + t * ldq + (long)h * head_stride;
+  const float u = ld_f(src + 2 * pi), v = ld_f(src + 2 * pi + 1);
+  float sn, cs;
+  sincosf((float)tok_pos[t] * inv_freq[pi], &sn, &cs);
+  float* dst = out + t * ldo + (long)h * out_head_stride;
+  dst[2 * pi] = u * cs - v * sn;
+  dst[2 * pi + 1] = v * cs + u * sn;
+}
+
+// workgroup = (token, head): one key per lane and tile for the scores, one value dimension per lane for the weighted sum
+template <typename T, int NACC>
+__global__ __launch_bounds__(256) void latent_attn_kernel(const float* __restrict__ q, const T* __restrict__ pool,
+                                                          const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+                                                          const int* __restrict__ block_table, int max_pages, int H, int R, int Dr,
+                                                          float scale, const T* __restrict__ gate, long ldgate,
+                                                          float* __restrict__ out) {
+  extern __shared__ float smem[];
+  const int Dk = R + Dr;
+  float* qs = smem;              // [Dk]
+  float* ps = qs + Dk;           // [256]
+  float* red = ps + 256;         // [8]
+  const long t = blockIdx.x;
+  const int h = blockIdx.y, tid = threadIdx.x;
+  const int pos = tok_pos[t];
+  const int* bt = block_table + (long)tok_seq[t] * max_pages;
+  for (int i = tid; i < Dk; i += 256) qs[i] = q[(t * H + h) * Dk + i];
+  __syncthreads();
+  float m_run = -INFINITY, l_run = 0.f;
+  float acc[NACC];
+#pragma unroll
+  for (int a = 0; a < NACC; ++a) acc[a] = 0.f;
+  const int nkeys = pos + 1;
+  for (int j0 = 0; j0 < nkeys; j0 += 256) {
+    const int j = j0 + tid;
+    float s = -INFINITY;
+    if (j < nkeys) {
+      const T* kr = pool + ((long)bt[j / PAGE] * PAGE + j % PAGE) * Dk;
+      float d = 0.f;
+      for (int i = 0; i < Dk; ++i) d = fmaf(qs[i], ld_f(kr + i), d);
+      s = d * scale;
+    }
+    float mx = s;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    if ((tid & 63) == 0) red[tid >> 6] = mx;
+    __syncthreads();
+    const float m_new = fmaxf(m_run, fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])));
+    const float pj = j < nkeys ? expf(s - m_new) : 0.f;
+    ps[tid] = pj;
+    float sum = pj;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+    if ((tid & 63) == 0) red[4 + (tid >> 6)] = sum;
+    __syncthreads();
+    const float alpha = expf(m_run - m_new);           // (first tile: exp(-inf) = 0)
+    l_run = l_run * alpha + ((red[4] + red[5]) + (red[6] + red[7]));
+    m_run = m_new;
+    const int nk = min(256, nkeys - j0);
+#pragma unroll
+    for (int a = 0; a < NACC; ++a) {
+      const int dcol = tid + a * 256;
+      if (dcol < R) {
+        float v = acc[a] * alpha;
+        for (int jj = 0; jj < nk; ++jj) {
+          const int key = j0 + jj;
+          v = fmaf(ps[jj], ld_f(pool + ((long)bt[key / PAGE] * PAGE + key % PAGE) * Dk + dcol), v);
+        }
+        acc[a] = v;
+      }
+    }
+    __syncthreads();
+  }
+  float gsc = 1.f / l_run;
+  if (gate) gsc *= 1.f / (1.f + expf(-ld_f(gate + t * ldgate + h)));
+#pragma unroll
+  for (int a = 0; a < NACC; ++a) {
+    const int dcol = tid + a * 256;
+    if (dcol < R) out[(t * H + h) * R + dcol] = acc[a] * gsc;
+  }
+}
+
+}  // namespace
+
+extern "C" int vlm_latent_kv_write(const void* d, long ldd, const void* w, int R, int Dr, const void* inv_freq, const void* tok_seq,
+                                   const void* tok_pos, const void* block_table, int max_pages, void* pool, float eps, int rows,
+                                   int dtype, void* stream) {
+  if (!d || !w || !tok_seq || !tok_pos || !block_table || !pool || R <= 0 || Dr < 0 || (Dr & 1) || (Dr && !inv_freq) ||
+      ldd < R + Dr || max_pages <= 0 || rows < 0)
+    return VLM_ERR_ARG;
+  if (rows == 0) return VLM_OK;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype)
+    hipLaunchKernelGGL(latent_kv_write_kernel<float>, dim3(rows), dim3(256), 0, st, (const float*)d, ldd, (const float*)w, R, Dr,
+                       (const float*)inv_freq, (const int*)tok_seq, (const int*)tok_pos, (const int*)block_table, max_pages,
+                       (float*)pool, eps);
+  else
+    hipLaunchKernelGGL(latent_kv_write_kernel<bf16_t>, dim3(rows), dim3(256), 0, st, (const bf16_t*)d, ldd, (const bf16_t*)w, R, Dr,
+                       (const float*)inv_freq, (const int*)tok_seq, (const int*)tok_pos, (const int*)block_table, max_pages,
+                       (bf16_t*)pool, eps);
+  VLM_CHECK_LAUNCH();
+  return VLM_OK;
+}
+
+extern "C" int vlm_rope_pairs_rows(const void* q, long ldq, long head_stride, int H, int Dr, const void* inv_freq, const void* tok_pos,
+                                   void* out, long ldo, long out_head_stride, int rows, int dtype, void* stream) {
+  if (!q || !tok_pos || !out || H <= 0 || Dr < 0 || (Dr & 1) || (Dr && !inv_freq) || rows < 0) return VLM_ERR_ARG;
+  if (rows == 0 || Dr == 0) return VLM_OK;
+  hipStream_t st = (hipStream_t)stream;
+  const unsigned nb = (unsigned)(((long)rows * H * (Dr / 2) + 255) / 256);
+  if (dtype)
+    hipLaunchKernelGGL(rope_pairs_rows_kernel<float>, dim3(nb), dim3(256), 0, st, (const float*)q, ldq, head_stride, H, Dr,
+                       (const float*)inv_freq, (const int*)tok_pos, (float*)out, ldo, out_head_stride, rows);
+  else
+    hipLaunchKernelGGL(rope_pairs_rows_kernel<bf16_t>, dim3(nb), dim3(256), 0, st, (const bf16_t*)q, ldq, head_stride, H, Dr,
+                       (const float*)inv_freq, (const int*)tok_pos, (float*)out, ldo, out_head_stride, rows);
+  VLM_CHECK_LAUNCH();
+  return VLM_OK;
+}
+
+extern "C" int vlm_latent_attn(const void* q, const void* pool, const void* tok_seq, const void* tok_pos, const void* block_table,
+                               int max_pages, int H, int R, int Dr, float scale, const void* gate, long ldgate, void* out, int rows,
+                               int dtype, void* stream) {
+  if (!q || !pool || !tok_seq || !tok_pos || !block_table || !out || H <= 0 || R <= 0 || Dr < 0 || max_pages <= 0 || rows < 0 ||
+      (gate && ldgate < H))
+    return VLM_ERR_ARG;
+  if (rows == 0) return VLM_OK;
+  if (R > 1024 || H > 65535) return VLM_ERR_SHAPE;
+  hipStream_t st = (hipStream_t)stream;
+  const size_t lds = (size_t)(R + Dr + 256 + 8) * sizeof(float);
+  dim3 grid(rows, H);
+#define GO(T, N)                                                                                                                  \
+  hipLaunchKernelGGL((latent_attn_kernel<T, N>), grid, dim3(256), lds, st, (const float*)q, (const T*)pool, (const int*)tok_seq,  \
+                     (const int*)tok_pos, (const int*)block_table, max_pages, H, R, Dr, scale, (const T*)gate, ldgate, (float*)out)
+  const int nacc = (R + 255) / 256;
+  if (dtype) {
+    if (nacc == 1) GO(float, 1); else if (nacc == 2) GO(float, 2); else GO(float, 4);
+  } else {
+    if (nacc == 1) GO(bf16_t, 1); else if (nacc == 2) GO(bf16_t, 2); else GO(bf16_t, 4);
+  }
+#undef GO
+  VLM_CHECK_LAUNCH();
+  return VLM_OK;
+}

@@ -1,0 +1,152 @@
+// Generic strided, batched linear layer for the shapes and number formats the MFMA GEMMs (gemm_bf16.hip) do not take:
+//
+//     C[b][m][n] (+)= sum_k A[b][m][k] * W[b][n][k]          b < batch, any M, N, K, any leading dimension
+//
+// A, W and C are each bf16 or fp32 (codes 0 / 1); products and sums are fp32 FMAs in ascending k, so a row of C depends on
+// nothing but its own row of A: the result of a token is the same bits whatever else is in the batch and however a
+// prompt was cut into steps.  With all three in fp32 this is the true 32-bit product of the float32 serving mode; with
+// fp32 C and `accumulate` it adds a projection straight onto an fp32 residual stream.
+//
+// 64 x 64 output tile per workgroup of 256 lanes (4 waves), 16-deep k slabs staged through LDS as fp32, 4 x 4 outputs
+// per lane.  Per-head projections of one tensor (latent attention's absorbed key / value maps) run as `batch` with
+// element strides between heads.
+#include "common.hpp"
+#include "../../include/vlm_hip.h"
+
+namespace {
+
+template <typename T> __device__ __forceinline__ float ld_f(const T* p);
+template <> __device__ __forceinline__ float ld_f<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float ld_f<bf16_t>(const bf16_t* p) { return bf2f(*p); }
+template <typename T> __device__ __forceinline__ void st_f(T* p, float v);
+template <> __device__ __forceinline__ void st_f<float>(float* p, float v) { *p = v; }
+template <> __device__ __forceinline__ void st_f<bf16_t>(bf16_t* p, float v) { *p = f2bf(v); }
+
+constexpr int BM = 64, BN = 64, BK = 16;
+
+template <typename TA, typename TW, typename TC>
+__global__ __launch_bounds__(256) void linear_any_kernel(const TA* __restrict__ A, const TW* __restrict__ W, TC* __restrict__ C,
+                                                         int M, int N, int K, long lda, long ldw, long ldc, long sA, long sW,
+                                                         long sC, int accumulate) {
+  __shared__ float As[BK][BM + 4];
+  __shared__ float Ws[BK][BN + 4];
+  const int b = blockIdx.z;
+  A += (long)b * sA;
+  W += (long)b * sW;
+  C += (long)b * sC;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const int tid = threadIdx.x;
+  const int tm = (tid / 16) * 4, tn = (tid % 16) * 4;
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    // 64 rows x 16 k of each operand: lane -> (row = tid / 4, 4 consecutive k)
+    const int r = tid >> 2, kk = (tid & 3) * 4;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int k = k0 + kk + j;
+      As[kk + j][r] = (m0 + r < M && k < K) ? ld_f(A + (long)(m0 + r) * lda + k) : 0.f;
+      Ws[kk + j][r] = (n0 + r < N && k < K) ? ld_f(W + (long)(n0 + r) * ldw + k) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < BK; ++k) {
+      float a[4], w[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = As[k][tm + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) w[j] = Ws[k][tn + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = m0 + tm + i;
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tn + j;
+      if (n >= N) continue;
+      TC* c = C + (long)m * ldc + n;
+      st_f(c, accumulate ? ld_f(c) + acc[i][j] : acc[i][j]);
+    }
+  }
+}
+
+// few rows (decode steps): the weights are the traffic, so W is read ONCE for all rows.  One wave per output column, lanes
+// across k (coalesced), up to 8 row accumulators per lane, xor-butterfly sum: a fixed order, so a row's result is still a
+// function of that row alone.  Sum order differs from the tile kernel's (rounding only).
+template <typename TA, typename TW, typename TC>
+__global__ __launch_bounds__(256) void linear_rows_kernel(const TA* __restrict__ A, const TW* __restrict__ W, TC* __restrict__ C,
+                                                          int M, int N, int K, long lda, long ldw, long ldc, long sA, long sW,
+                                                          long sC, int accumulate) {
+  const int b = blockIdx.z;
+  A += (long)b * sA;
+  W += (long)b * sW;
+  C += (long)b * sC;
+  const int n = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (n >= N) return;                                     // (whole waves leave together: n is uniform per wave)
+  const TW* w = W + (long)n * ldw;
+  float acc[8] = {};
+  for (int k = lane; k < K; k += 64) {
+    const float wv = ld_f(w + k);
+#pragma unroll
+    for (int m = 0; m < 8; ++m)
+      if (m < M) acc[m] = fmaf(ld_f(A + (long)m * lda + k), wv, acc[m]);
+  }
+#pragma unroll
+  for (int m = 0; m < 8; ++m) {
+    if (m >= M) break;
+    float v = acc[m];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    if (lane == 0) {
+      TC* c = C + (long)m * ldc + n;
+      st_f(c, accumulate ? ld_f(c) + v : v);
+    }
+  }
+}
+
+template <typename TA, typename TW, typename TC>
+int launch(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc, int batch, long sA, long sW,
+           long sC, int accumulate, hipStream_t st) {
+  if (M <= 8) {
+    dim3 grid((N + 3) / 4, 1, batch);
+    hipLaunchKernelGGL((linear_rows_kernel<TA, TW, TC>), grid, dim3(256), 0, st, (const TA*)A, (const TW*)W, (TC*)C, M, N, K, lda,
+                       ldw, ldc, sA, sW, sC, accumulate);
+  } else {
+    dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM, batch);
+    hipLaunchKernelGGL((linear_any_kernel<TA, TW, TC>), grid, dim3(256), 0, st, (const TA*)A, (const TW*)W, (TC*)C, M, N, K, lda,
+                       ldw, ldc, sA, sW, sC, accumulate);
+  }
+  VLM_CHECK_LAUNCH();
+  return VLM_OK;
+}
+
+}  // namespace
+
+extern "C" int vlm_linear_any(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc, int a_f32,
+                              int w_f32, int c_f32, int batch, long strideA, long strideW, long strideC, int accumulate,
+                              void* stream) {
+  if (!A || !W || !C || M < 0 || N <= 0 || K <= 0 || batch <= 0 || lda < K || ldw < K || ldc < N) return VLM_ERR_ARG;
+  if (accumulate && !c_f32) return VLM_ERR_ARG;
+  if (M == 0) return VLM_OK;
+  if (M > 65535 * 64 || batch > 65535) return VLM_ERR_SHAPE;
+  hipStream_t st = (hipStream_t)stream;
+  const int code = (a_f32 ? 4 : 0) | (w_f32 ? 2 : 0) | (c_f32 ? 1 : 0);
+#define GO(TA, TW, TC) return launch<TA, TW, TC>(A, W, C, M, N, K, lda, ldw, ldc, batch, strideA, strideW, strideC, accumulate, st)
+  switch (code) {
+    case 0: GO(bf16_t, bf16_t, bf16_t);
+    case 1: GO(bf16_t, bf16_t, float);
+    case 2: GO(bf16_t, float, bf16_t);
+    case 3: GO(bf16_t, float, float);
+    case 4: GO(float, bf16_t, bf16_t);
+    case 5: GO(float, bf16_t, float);
+    case 6: GO(float, float, bf16_t);
+    default: GO(float, float, float);
+  }
+#undef GO
+}

@@ -1,0 +1,238 @@
+// Matrix-state linear recurrences (linear attention without softmax), carried per sequence in fp32:
+//
+//     S_t = a_t * S_(t-1) + b_t * k_t v_t^T            o_t = S_t^T q_t                      S: [D, Dv] per head
+//
+//   * fixed decay ("retention"): a_t = decay[h], b_t = 1, rotary positions on q and k (rotate-half pairing on the first
+//     rot_dims dimensions), k scaled after the rotation;
+//   * gated ("mLSTM"): log input gate i_t = cap * tanh((i~ + bias) / cap), log forget gate f_t = logsigmoid(cap * tanh((f~ +
+//     bias) / cap)), running maximum m_t = max(f_t + m_(t-1), i_t) with m_0 = 0, a_t = exp(f_t + m_(t-1) - m_t),
+//     b_t = exp(i_t - m_t); the normaliser n_t = a_t n_(t-1) + b_t k_t rides along as one more COLUMN of S (v extended by a
+//     constant 1), so n_t . q_t is one more output; o_t is divided by max(|n_t . q_t|, exp(-m_t)) + 1e-6.
+//
+// One kernel serves a whole prompt, a portion of one and a single decoded token: a segment is `len` consecutive tokens of one
+// sequence; its state is read from the sequence's slot (zero when the segment starts at position 0 - a slot that is used
+// again needs no clearing), advanced token by token with the same arithmetic wherever the prompt was cut, and written back.
+// vlm_linear_recurrence writes the raw o (and n . q) in fp32; vlm_recurrence_finish then applies the denominator, the
+// per-head unit-RMS norm, an optional weight and the output gate (silu or sigmoid of a projection) into a T-typed row.
+//
+// Work split: workgroup = (segment, head, tile of 64 state columns); lane c of part p holds rows [32 p, 32 p + 32) of column
+// c in registers.  Tokens are staged 4 / 8 / 16 at a time through LDS (q, k rotated and scaled on the way in).
+#include "common.hpp"
+#include "../../include/vlm_hip.h"
+
+namespace {
+
+template <typename T> __device__ __forceinline__ float ld_f(const T* p);
+template <> __device__ __forceinline__ float ld_f<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float ld_f<bf16_t>(const bf16_t* p) { return bf2f(*p); }
+template <typename T> __device__ __forceinline__ void st_f(T* p, float v);
+template <> __device__ __forceinline__ void st_f<float>(float* p, float v) { *p = v; }
+template <> __device__ __forceinline__ void st_f<bf16_t>(bf16_t* p, float v) { *p = f2bf(v); }
+
+constexpr int DR = 32;       // state rows per lane
+constexpr int CT = 64;       // state columns per workgroup
+
+__device__ __forceinline__ float logsigmoid_f(float x) { return fminf(x, 0.f) - log1pf(expf(-fabsf(x))); }
+
+template <typename T, bool GATED>
+__global__ __launch_bounds__(1024) void linear_recurrence_kernel(vlm_recurrence_args p, int P, int TB) {
+  extern __shared__ float smem[];
+  const int seg = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * CT;
+  const int D = p.D, Dv = p.Dv, C = Dv + (GATED ? 1 : 0), DP = P * DR;
+  const int tid = threadIdx.x, nthr = blockDim.x;
+  const int part = tid / CT, col = c0 + (tid % CT), row0 = part * DR;
+  float* qs = smem;                       // [TB][DP]
+  float* ks = qs + TB * DP;               // [TB][DP]
+  float* vs = ks + TB * DP;               // [TB][CT]
+  float* ab = vs + TB * CT;               // [TB][4]: a, b, (gated) i, f / scratch
+  float* po = ab + TB * 4;                // [TB][P][CT]
+  const int t_begin = p.seg_start[seg], t_end = p.seg_start[seg + 1];
+  const int slot = p.seg_slot[seg], pos0 = p.seg_pos0[seg];
+  const T* q = (const T*)p.q + (long)h * D;
+  const T* k = (const T*)p.k + (long)h * D;
+  const T* v = (const T*)p.v + (long)h * Dv;
+  float* S = p.state + ((long)slot * p.H + h) * (long)D * C;
+  float s[DR];
+#pragma unroll
+  for (int r = 0; r < DR; ++r) {
+    const int row = row0 + r;
+    s[r] = (pos0 > 0 && row < D && col < C) ? S[(long)row * C + col] : 0.f;
+  }
+  // (GATED: meaningful in lane 0; the maximum the segment starts from was saved by gate_max_kernel, which has already
+  //  moved the slot's own value to the end of the segment - every column tile must see the OLD one)
+  float m_run = GATED ? p.mprev[(long)seg * p.H + h] : 0.f;
+  const int half = p.rot_dims / 2;
+  const float dec = GATED ? 0.f : p.decay[h];
+
+  for (int t0 = t_begin; t0 < t_end; t0 += TB) {
+    const int nb = min(TB, t_end - t0);
+    for (int idx = tid; idx < nb * DP; idx += nthr) {
+      const int t = idx / DP, i = idx % DP;
+      float qv = 0.f, kv = 0.f;
+      if (i < D) {
+        const long tok = t0 + t;
+        qv = ld_f(q + tok * p.ldq + i);
+        kv = ld_f(k + tok * p.ldk + i);
+        if (i < p.rot_dims) {
+          const int j = i < half ? i + half : i - half;
+          const float ang = (float)(pos0 + (t0 - t_begin) + t) * p.inv_freq[i < half ? i : i - half];
+          float sn, cs;
+          sincosf(ang, &sn, &cs);
+          const float qo = ld_f(q + tok * p.ldq + j), ko = ld_f(k + tok * p.ldk + j);
+          // (u, v) -> (u cos - v sin, v cos + u sin): the first half holds u, the second v
+          qv = i < half ? qv * cs - qo * sn : qv * cs + qo * sn;
+          kv = i < half ? kv * cs - ko * sn : kv * cs + ko * sn;
+        }
+        qv *= p.qscale;
+        kv *= p.kscale;
+      }
+      qs[idx] = qv;
+      ks[idx] = kv;
+    }
+    for (int idx = tid; idx < nb * CT; idx += nthr) {
+      const int t = idx / CT, c = c0 + idx % CT;
+      vs[idx] = c < Dv ? ld_f(v + (long)(t0 + t) * p.ldv + c) : (c == Dv && GATED ? 1.f : 0.f);
+    }
+    if (GATED) {
+      if (tid < nb) {
+        const long tok = t0 + tid;
+        const float iv = ld_f((const T*)p.ipre + tok * p.ldi + h) + ld_f((const T*)p.ib + h);
+        const float fv = ld_f((const T*)p.fpre + tok * p.ldf + h) + ld_f((const T*)p.fb + h);
+        ab[tid * 4 + 2] = p.cap * tanhf(iv / p.cap);
+        ab[tid * 4 + 3] = logsigmoid_f(p.cap * tanhf(fv / p.cap));
+      }
+      __syncthreads();
+      if (tid == 0) {                     // the scalar scan: adds and maxima only; the exponentials follow in parallel
+        for (int t = 0; t < nb; ++t) {
+          const float ig = ab[t * 4 + 2], fg = ab[t * 4 + 3];
+          const float m_new = fmaxf(fg + m_run, ig);
+          ab[t * 4 + 0] = fg + m_run - m_new;
+          ab[t * 4 + 1] = ig - m_new;
+          m_run = m_new;
+        }
+      }
+      __syncthreads();
+      if (tid < nb) {
+        ab[tid * 4 + 0] = expf(ab[tid * 4 + 0]);
+        ab[tid * 4 + 1] = expf(ab[tid * 4 + 1]);
+      }
+    }
+    __syncthreads();
+    for (int t = 0; t < nb; ++t) {
+      const float a = GATED ? ab[t * 4 + 0] : dec, b = GATED ? ab[t * 4 + 1] : 1.f;
+      const float bv = b * vs[t * CT + (tid % CT)];
+      const float* kr = ks + t * DP + row0;
+      const float* qr = qs + t * DP + row0;
+      float acc = 0.f;
+#pragma unroll
+      for (int r = 0; r < DR; ++r) {
+        s[r] = fmaf(a, s[r], kr[r] * bv);
+        acc = fmaf(s[r], qr[r], acc);
+      }
+      po[(t * P + part) * CT + (tid % CT)] = acc;
+    }
+    __syncthreads();
+    for (int idx = tid; idx < nb * CT; idx += nthr) {
+      const int t = idx / CT, cc = idx % CT;
+      if (c0 + cc < C) {
+        float o = 0.f;
+        for (int pp = 0; pp < P; ++pp) o += po[(t * P + pp) * CT + cc];
+        p.raw[((long)(t0 + t) * p.H + h) * C + c0 + cc] = o;
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int r = 0; r < DR; ++r) {
+    const int row = row0 + r;
+    if (row < D && col < C) S[(long)row * C + col] = s[r];
+  }
+}
+
+// the running maximum m_t per (token, head) for the finish pass, and the slot's maximum moved to the end of the segment:
+// the same scan as above, one lane per (segment, head)
+template <typename T>
+__global__ void gate_max_kernel(vlm_recurrence_args p, int nseg) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= nseg * p.H) return;
+  const int seg = i / p.H, h = i % p.H;
+  float* ms = p.mstate + (long)p.seg_slot[seg] * p.H + h;
+  float m = p.seg_pos0[seg] > 0 ? *ms : 0.f;
+  p.mprev[i] = m;
+  for (int tok = p.seg_start[seg]; tok < p.seg_start[seg + 1]; ++tok) {
+    const float iv = ld_f((const T*)p.ipre + (long)tok * p.ldi + h) + ld_f((const T*)p.ib + h);
+    const float fv = ld_f((const T*)p.fpre + (long)tok * p.ldf + h) + ld_f((const T*)p.fb + h);
+    m = fmaxf(logsigmoid_f(p.cap * tanhf(fv / p.cap)) + m, p.cap * tanhf(iv / p.cap));
+    p.mtok[(long)tok * p.H + h] = m;
+  }
+  *ms = m;
+}
+
+template <typename T, bool GATED>
+__global__ __launch_bounds__(64) void recurrence_finish_kernel(vlm_recurrence_args p) {
+  const long tok = blockIdx.x;
+  const int h = blockIdx.y, lane = threadIdx.x;
+  const int Dv = p.Dv, C = Dv + (GATED ? 1 : 0);
+  const float* o = p.raw + (tok * p.H + h) * C;
+  float inv = 1.f;
+  if (GATED) inv = 1.f / (fmaxf(fabsf(o[Dv]), expf(-p.mtok[tok * p.H + h])) + 1e-6f);
+  float ss = 0.f;
+  for (int c = lane; c < Dv; c += 64) {
+    const float x = o[c] * inv;
+    ss += x * x;
+  }
+#pragma unroll
+  for (int d = 32; d > 0; d >>= 1) ss += __shfl_xor(ss, d);
+  const float r = 1.0f / sqrtf(ss / (float)Dv + p.eps);
+  const T* g = (const T*)p.g + tok * p.ldg + (long)h * Dv;
+  T* out = (T*)p.out + tok * p.ldo + (long)h * Dv;
+  for (int c = lane; c < Dv; c += 64) {
+    float x = o[c] * inv * r;
+    if (p.normw) x *= ld_f((const T*)p.normw + (long)h * Dv + c);
+    const float gv = ld_f(g + c), sg = 1.f / (1.f + expf(-gv));
+    st_f(out + c, x * (p.gate_act == 0 ? gv * sg : sg));
+  }
+}
+
+template <typename T>
+int run(const vlm_recurrence_args& a, int nseg, int ntok, hipStream_t st) {
+  const int gated = a.gated;
+  const int C = a.Dv + (gated ? 1 : 0);
+  const int P = (a.D + DR - 1) / DR;
+  if (P * CT > 1024) return VLM_ERR_SHAPE;
+  int TB = 16;
+  auto lds = [&](int tb) { return (size_t)tb * (2 * P * DR + CT + 4 + P * CT) * sizeof(float); };
+  while (TB > 4 && lds(TB) > 48 * 1024) TB >>= 1;
+  if (lds(TB) > 64 * 1024) return VLM_ERR_SHAPE;
+  dim3 grid(nseg, a.H, (C + CT - 1) / CT), block(P * CT);
+  if (gated) {
+    // the per-token maxima first: the scan kernel overwrites the slot's running maximum
+    hipLaunchKernelGGL(gate_max_kernel<T>, dim3((nseg * a.H + 63) / 64), dim3(64), 0, st, a, nseg);
+    VLM_CHECK_LAUNCH();
+    hipLaunchKernelGGL((linear_recurrence_kernel<T, true>), grid, block, lds(TB), st, a, P, TB);
+  } else {
+    hipLaunchKernelGGL((linear_recurrence_kernel<T, false>), grid, block, lds(TB), st, a, P, TB);
+  }
+  VLM_CHECK_LAUNCH();
+  if (gated) hipLaunchKernelGGL((recurrence_finish_kernel<T, true>), dim3(ntok, a.H), dim3(64), 0, st, a);
+  else hipLaunchKernelGGL((recurrence_finish_kernel<T, false>), dim3(ntok, a.H), dim3(64), 0, st, a);
+  VLM_CHECK_LAUNCH();
+  return VLM_OK;
+}
+
+}  // namespace
+
+extern "C" int vlm_linear_recurrence(const vlm_recurrence_args* a, int nseg, int ntok, int dtype, void* stream) {
+  if (!a || nseg < 0 || ntok < 0) return VLM_ERR_ARG;
+  if (!a->q || !a->k || !a->v || !a->g || !a->state || !a->raw || !a->out || !a->seg_start || !a->seg_slot || !a->seg_pos0)
+    return VLM_ERR_ARG;
+  if (a->H <= 0 || a->D <= 0 || a->Dv <= 0 || a->rot_dims < 0 || a->rot_dims > a->D || (a->rot_dims & 1)) return VLM_ERR_ARG;
+  if (a->rot_dims && !a->inv_freq) return VLM_ERR_ARG;
+  if (a->gated ? (!a->ipre || !a->fpre || !a->ib || !a->fb || !a->mstate || !a->mtok || !a->mprev || !(a->cap > 0.f)) : !a->decay) return VLM_ERR_ARG;
+  if (a->ldq < (long)a->H * a->D || a->ldk < (long)a->H * a->D || a->ldv < (long)a->H * a->Dv || a->ldg < (long)a->H * a->Dv ||
+      a->ldo < (long)a->H * a->Dv)
+    return VLM_ERR_ARG;
+  if (nseg == 0 || ntok == 0) return VLM_OK;
+  if (nseg > 65535 * 16 || a->H > 65535) return VLM_ERR_SHAPE;
+  return dtype ? run<float>(*a, nseg, ntok, (hipStream_t)stream) : run<bf16_t>(*a, nseg, ntok, (hipStream_t)stream);
+}

@@ -391,6 +391,8 @@ def generate_step(input_ids, model, pixel_values, mask, *, max_tokens: int = DEF
     base_offset = seq.offset
 
     lookahead = max(1, min(int(lookahead), st.ring_len - 1))
+    if getattr(lm, "STATEFUL", False):
+        lookahead = 0        # recurrent state cannot be rolled back: no step is enqueued before its token is asked for
     pipe = _TokenPipe(1, cap=lookahead + 2)
     pipe.push(0, tok0)
     lps: List[Optional[torch.Tensor]] = [lp0[0] if lp0 is not None else None] + [None] * (lookahead + 1)

@@ -632,3 +632,121 @@ def make_prompt_cache(model, max_kv_size: Optional[int] = None):
     if max_kv_size is not None:
         caches[0]._seq.set_rotating(int(max_kv_size), keep=4)
     return caches
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# Hybrid models: layers that cache ONE row per token (latent attention) next to layers that carry a fixed-size recurrent
+# state per sequence (the reference keeps such states in ArraysCache / MambaCache objects, cache.py:628-760, one per layer and
+# request).  Here both live in one pool object: the row caches share the page allocator and the block table of KVPool (page =
+# 64 tokens, any row width, bf16 or fp32), the states are indexed by the SAME sequence slot as the block-table row - a request
+# that ends gives back its pages and its slot together, and the next request that takes the slot starts from a zero state
+# because the recurrence kernels ignore the stored state of a segment that begins at position 0 (nothing is cleared).
+class HybridPool(KVPool):
+    def __init__(self, n_layers: int, row_layers, state_layers, max_tokens: int, max_seqs: int, device="cuda",
+                 dtype=torch.bfloat16, max_pages_per_seq: Optional[int] = None):
+        """row_layers: {layer: row width} for layers that write one cached row per token;
+        state_layers: {layer: (heads, rows, cols, has_scalar)}: fp32 state [heads, rows, cols] (+ one fp32 scalar per head)"""
+        self.n_layers = n_layers
+        self.n_kv_heads = self.head_dim = 0                    # (no per-head K / V pages in this pool)
+        self.n_pages = (max_tokens + PAGE - 1) // PAGE
+        self.max_seqs = max_seqs
+        self.max_pages = max_pages_per_seq or self.n_pages
+        self.identity = False
+        self.device = device
+        self.dtype = dtype
+        self.rows = {int(l): torch.zeros(self.n_pages, PAGE, int(w), dtype=dtype, device=device) for l, w in row_layers.items()}
+        self.state = {int(l): torch.zeros(max_seqs, h, r, c, dtype=torch.float32, device=device)
+                      for l, (h, r, c, _) in state_layers.items()}
+        self.scalar = {int(l): torch.zeros(max_seqs, h, dtype=torch.float32, device=device)
+                       for l, (h, r, c, sc) in state_layers.items() if sc}
+        self.kpool = self.vpool = None
+        self.layer_stride = 0
+        self.block_table_host = np.zeros((max_seqs, self.max_pages), dtype=np.int32)
+        self.block_table = torch.zeros(max_seqs, self.max_pages, dtype=torch.int32, device=device)
+        self._free_pages = list(range(self.n_pages - 1, -1, -1))
+        self._free_seqs = set(range(max_seqs))
+
+    @property
+    def nbytes(self):
+        return sum(t.numel() * t.element_size() for d in (self.rows, self.state, self.scalar) for t in d.values())
+
+    @property
+    def free_pages(self) -> int:
+        return len(self._free_pages)
+
+    def ensure_q8(self):
+        raise NotImplementedError("quantized KV cache: not built for row / state caches")
+
+    def layer_views(self, layer: int):
+        raise NotImplementedError("HybridPool holds rows and states, not per-head K / V pages")
+
+
+class RowCache:
+    """Per-layer facade of a layer that caches one row per token (latent attention): the reference's cache attributes that
+    make sense for it (`offset`, `state`, `trim`)."""
+
+    def __init__(self, seq: PagedSequence, layer: int):
+        self._seq, self._layer = seq, layer
+
+    @property
+    def offset(self):
+        return self._seq.offset
+
+    def empty(self):
+        return self._seq.offset == 0
+
+    def size(self):
+        return self._seq.offset
+
+    def is_trimmable(self):
+        return True
+
+    def trim(self, n):
+        n = min(self._seq.offset, n)
+        if self._layer == min(self._seq.pool.rows):
+            self._seq.set_offset(self._seq.offset - n)
+        return n
+
+    @property
+    def state(self):
+        """the cached rows [offset, width] in token order (debug / interop)"""
+        s, pool = self._seq, self._seq.pool
+        pages = torch.as_tensor(s.pages[: (s.offset + PAGE - 1) // PAGE], dtype=torch.long, device=pool.block_table.device)
+        return pool.rows[self._layer][pages].reshape(-1, pool.rows[self._layer].shape[-1])[: s.offset]
+
+    @property
+    def nbytes(self):
+        t = self._seq.pool.rows[self._layer]
+        return len(self._seq.pages) * PAGE * t.shape[-1] * t.element_size()
+
+
+class RecurrentCache:
+    """Per-layer facade of a recurrent layer's state slot (reference ArraysCache, cache.py:628-700: `state`, not trimmable)."""
+
+    def __init__(self, seq: PagedSequence, layer: int):
+        self._seq, self._layer = seq, layer
+
+    @property
+    def offset(self):
+        return self._seq.offset
+
+    def empty(self):
+        return self._seq.offset == 0
+
+    def is_trimmable(self):
+        return False                          # a recurrence cannot forget its last tokens
+
+    def trim(self, n):
+        return 0
+
+    @property
+    def state(self):
+        pool, s = self._seq.pool, self._seq.seq
+        out = [pool.state[self._layer][s]]
+        if self._layer in pool.scalar:
+            out.append(pool.scalar[self._layer][s])
+        return out
+
+    @property
+    def nbytes(self):
+        return sum(t.numel() * t.element_size() for t in self.state)

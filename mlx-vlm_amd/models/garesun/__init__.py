@@ -1,0 +1,8 @@
+"""`models.garesun`: a decoder-only language model of heterogeneous layers - matrix-state recurrences (fixed-decay
+retention, gated mLSTM) and latent attention, each in parallel with a mixture-of-experts feed-forward, plus a per-layer
+token input - with the module contract of the other model packages (ModelConfig / Model / LanguageModel)."""
+from .config import LayerConfig, ModelConfig
+from .garesun import Model
+from .language import LanguageModel
+
+__all__ = ["Model", "ModelConfig", "LayerConfig", "LanguageModel"]

@@ -546,3 +546,130 @@ def dequant_w4(wq, sb, rows=None, out=None):
 def gemm_set_staging(mode: int):
     """0 = automatic (LDS DMA when K % 64 == 0), 1 = always register staging (test / A-B knob)."""
     check(_lib.lib().vlm_gemm_set_staging(int(mode)), "gemm_set_staging")
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# Operators of decoders with an fp32 residual stream (include/vlm_hip.h, second part).  "T" tensors are bf16 or fp32
+# (dtype code 0 / 1 of the C ABI, taken from the tensor); the stream x and every statistic are fp32.
+def _f32(t) -> int:
+    if t.dtype == torch.float32:
+        return 1
+    if t.dtype == torch.bfloat16:
+        return 0
+    raise _lib.VlmHipError(f"bf16 or fp32 tensor expected, got {t.dtype}")
+
+
+def linear_any(a, w, out=None, out_dtype=None, accumulate=False, batch=1, stride_a=0, stride_w=0, stride_c=0, M=None, N=None, K=None):
+    """out[b][m][n] (+)= sum_k a[b][m][k] w[b][n][k] (vlm_linear_any).  Plain call: a [M, K], w [N, K] -> out [M, N] of
+    out_dtype (default a's).  Batched call (per-head maps inside wider rows): pass M / N / K, `batch` and the element strides
+    between batch members; a / w / out are then 2-D views whose data_ptr is member 0 and whose stride(0) is the row pitch."""
+    _dev(a, w, out)
+    M = a.shape[0] if M is None else int(M)
+    K = a.shape[1] if K is None else int(K)
+    N = w.shape[0] if N is None else int(N)
+    if out is None:
+        out = torch.empty(M, N, dtype=out_dtype or a.dtype, device=a.device)
+    check(_lib.lib().vlm_linear_any(_p(a), _p(w), _p(out), M, N, K, a.stride(0), w.stride(0), out.stride(0), _f32(a), _f32(w),
+                                    _f32(out), int(batch), int(stride_a), int(stride_w), int(stride_c), int(bool(accumulate)),
+                                    _stream()), "linear_any")
+    return out
+
+
+def embed_scale_f32(ids, table, scale, out=None):
+    """x [T, D] fp32 = table[ids] * scale"""
+    _dev(ids, table, out)
+    T, D = ids.numel(), table.shape[1]
+    if out is None:
+        out = torch.empty(T, D, dtype=torch.float32, device=table.device)
+    check(_lib.lib().vlm_embed_scale_f32(_p(ids), _p(table), float(scale), _p(out), T, D, table.shape[0], _f32(table), _stream()),
+          "embed_scale_f32")
+    return out
+
+
+def layernorm_nobias(x, w, eps, out=None):
+    """LayerNorm with a weight and no bias over the fp32 stream x [T, D] -> T-typed (w's dtype)"""
+    _dev(x, w, out)
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise _lib.VlmHipError("layernorm_nobias: contiguous fp32 stream expected")
+    if out is None:
+        out = torch.empty(x.shape, dtype=w.dtype, device=x.device)
+    check(_lib.lib().vlm_layernorm_nobias(_p(x), _p(w), _p(out), x.shape[0], x.shape[1], out.stride(0), float(eps), _f32(w),
+                                          _stream()), "layernorm_nobias")
+    return out
+
+
+def stream_add_(x, a, b=None):
+    """x += a (+ b): fp32 stream x [T, D], T-typed a / b (views with a row pitch)"""
+    _dev(x, a, b)
+    check(_lib.lib().vlm_stream_add(_p(x), _p(a), a.stride(0), _p(b), b.stride(0) if b is not None else 0, x.shape[0], x.shape[1],
+                                    _f32(a), _stream()), "stream_add")
+    return x
+
+
+def unit_rms_add_(x, y, w, eps):
+    """x += y * rsqrt(mean(y^2) + eps) * w"""
+    _dev(x, y, w)
+    check(_lib.lib().vlm_unit_rms_add(_p(x), _p(y), y.stride(0), _p(w), x.shape[0], x.shape[1], float(eps), _f32(y), _stream()),
+          "unit_rms_add")
+    return x
+
+
+def gelu_tanh_gate_rows(g, table, ids, col0, out=None):
+    """out[t, j] = gelu_tanh(g[t, j]) * table[ids[t], col0 + j]"""
+    _dev(g, table, ids, out)
+    rows, dim = g.shape
+    if out is None:
+        out = torch.empty(rows, dim, dtype=g.dtype, device=g.device)
+    check(_lib.lib().vlm_gelu_tanh_gate_rows(_p(g), g.stride(0), _p(table), table.stride(0), _p(ids), int(col0), _p(out),
+                                             out.stride(0), rows, dim, table.shape[0], _f32(g), _stream()), "gelu_tanh_gate_rows")
+    return out
+
+
+def linear_recurrence(args: "_lib.RecurrenceArgs", nseg: int, ntok: int, dtype_f32: bool):
+    check(_lib.lib().vlm_linear_recurrence(C.byref(args), int(nseg), int(ntok), int(bool(dtype_f32)), _stream()), "linear_recurrence")
+
+
+def latent_kv_write(d, w, R, Dr, inv_freq, tok_seq, tok_pos, block_table, pool, eps):
+    """rows of d [T, >= R + Dr] -> (normed latent | rotated key part) at each token's (sequence, position) of the paged pool"""
+    _dev(d, w, inv_freq, tok_seq, tok_pos, block_table, pool)
+    check(_lib.lib().vlm_latent_kv_write(_p(d), d.stride(0), _p(w), int(R), int(Dr), _p(inv_freq), _p(tok_seq), _p(tok_pos),
+                                         _p(block_table), block_table.shape[1], _p(pool), float(eps), d.shape[0], _f32(d),
+                                         _stream()), "latent_kv_write")
+
+
+def rope_pairs_rows(q, head_stride, H, Dr, inv_freq, tok_pos, out, out_head_stride):
+    """interleaved-pair rotation of a Dr-wide part of every head: q / out are 2-D views at the part's first column"""
+    _dev(q, inv_freq, tok_pos, out)
+    check(_lib.lib().vlm_rope_pairs_rows(_p(q), q.stride(0), int(head_stride), int(H), int(Dr), _p(inv_freq), _p(tok_pos), _p(out),
+                                         out.stride(0), int(out_head_stride), q.shape[0], _f32(q), _stream()), "rope_pairs_rows")
+
+
+def latent_attn(q, pool, tok_seq, tok_pos, block_table, H, R, Dr, scale, gate=None, out=None):
+    """q fp32 [T, H, R + Dr] over the latent pool -> fp32 [T, H, R] (times sigmoid(gate[t, h]) when given)"""
+    _dev(q, pool, tok_seq, tok_pos, block_table, gate, out)
+    T = q.shape[0]
+    if out is None:
+        out = torch.empty(T, H, R, dtype=torch.float32, device=q.device)
+    check(_lib.lib().vlm_latent_attn(_p(q), _p(pool), _p(tok_seq), _p(tok_pos), _p(block_table), block_table.shape[1], int(H), int(R),
+                                     int(Dr), float(scale), _p(gate), gate.stride(0) if gate is not None else 0, _p(out), T,
+                                     _f32(pool), _stream()), "latent_attn")
+    return out
+
+
+def moe_route(logits, top):
+    """fp32 logits [T, E] -> (dense gate table fp32 [T, E], chosen indices int32 [T, top], their weights fp32 [T, top])"""
+    _dev(logits)
+    T, E = logits.shape
+    gate = torch.empty(T, E, dtype=torch.float32, device=logits.device)
+    idx = torch.empty(T, top, dtype=torch.int32, device=logits.device)
+    wgt = torch.empty(T, top, dtype=torch.float32, device=logits.device)
+    check(_lib.lib().vlm_moe_route(_p(logits), T, E, int(top), _p(gate), _p(idx), _p(wgt), _stream()), "moe_route")
+    return gate, idx, wgt
+
+
+def moe_relu2_gate(up, gate, E, ff, shared, out):
+    """out[t, c] = relu(up[t, c])^2 * gate[t, c // ff] over the E * ff expert columns, relu^2 alone over the `shared` ones"""
+    _dev(up, gate, out)
+    check(_lib.lib().vlm_moe_relu2_gate(_p(up), up.stride(0), _p(gate), int(E), int(ff), int(shared), _p(out), out.stride(0),
+                                        up.shape[0], _f32(up), _stream()), "moe_relu2_gate")
+    return out

@@ -37,7 +37,10 @@ MODEL_REMAPPING: Dict[str, str] = {
 
 def get_model_and_args(config: dict):
     """reference utils.py:588-635"""
-    model_type = config["model_type"].lower()
+    # (a checkpoint without `model_type` names its design under `architecture`)
+    model_type = str(config.get("model_type") or config.get("architecture") or "").lower()
+    if not model_type:
+        raise ValueError("config.json names no model_type / architecture")
     model_type = MODEL_REMAPPING.get(model_type, model_type)
     try:
         arch = importlib.import_module(f"{__package__}.models.{model_type}")
@@ -80,6 +83,8 @@ def read_sanitized_weights(model_path: str, model, config: dict) -> Dict[str, to
 
     Qz.check_quantization(config.get("quantization"))          # affine 4-bit / group 64 (utils.py:916-967)
     weights = model.sanitize(weights)
+    if getattr(model, "vision_tower", None) is None:           # text-only model
+        return weights
     vt = {k: v for k, v in weights.items() if k.startswith("vision_tower.")}
     vt = {"vision_tower." + k: v for k, v in model.vision_tower.sanitize(
         {k[len("vision_tower."):]: v for k, v in vt.items()}).items()}
