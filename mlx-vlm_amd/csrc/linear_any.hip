@@ -78,7 +78,7 @@ __global__ __launch_bounds__(256) void linear_any_kernel(const TA* __restrict__ 
 
 // few rows (decode steps): the weights are the traffic, so W is read ONCE for all rows.  One wave per output column, lanes
 // across k (coalesced), up to 8 row accumulators per lane, xor-butterfly sum: a fixed order, so a row's result is still a
-// function of that row alone.  Sum order differs from the tile kernel's (rounding only).
+// function of that row alone.  Sum order differs from the tile kernel's (rounding only); not used when everything is fp32.
 template <typename TA, typename TW, typename TC>
 __global__ __launch_bounds__(256) void linear_rows_kernel(const TA* __restrict__ A, const TW* __restrict__ W, TC* __restrict__ C,
                                                           int M, int N, int K, long lda, long ldw, long ldc, long sA, long sW,
@@ -113,7 +113,10 @@ __global__ __launch_bounds__(256) void linear_rows_kernel(const TA* __restrict__
 template <typename TA, typename TW, typename TC>
 int launch(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc, int batch, long sA, long sW,
            long sC, int accumulate, hipStream_t st) {
-  if (M <= 8) {
+  // all-fp32 operands (the float32 serving mode) always take the tile kernel: one summation order for every row count, so a
+  // token's result is the same bits in a prompt, in a portion and decoded alone
+  constexpr bool all_f32 = sizeof(TA) == 4 && sizeof(TW) == 4 && sizeof(TC) == 4;
+  if (M <= 8 && !all_f32) {
     dim3 grid((N + 3) / 4, 1, batch);
     hipLaunchKernelGGL((linear_rows_kernel<TA, TW, TC>), grid, dim3(256), 0, st, (const TA*)A, (const TW*)W, (TC*)C, M, N, K, lda,
                        ldw, ldc, sA, sW, sC, accumulate);

@@ -81,8 +81,9 @@ class DecodeRows:
         self.ctx = torch.zeros(B, dtype=i32, device=dev)
         self.step = torch.zeros(1, dtype=i32, device=dev)
         self.out_ring = torch.zeros(ring_len, B, dtype=i32, device=dev)
-        self.logits = torch.zeros(B, V, dtype=torch.bfloat16, device=dev)
-        self.logprobs = torch.zeros(B, V, dtype=torch.bfloat16, device=dev)
+        VL = _al8(V)           # row pitch: 16-byte aligned rows for any vocabulary
+        self.logits = torch.zeros(B, VL, dtype=torch.bfloat16, device=dev)[:, :V]
+        self.logprobs = torch.zeros(B, VL, dtype=torch.bfloat16, device=dev)[:, :V]
         self.seqs: List[PagedSequence] = []
         self.row_seqs: List[PagedSequence] = []
         self.graph_key = None
@@ -330,9 +331,11 @@ class LanguageModel:
             return None
         xl = x if rows.size == Tn and np.array_equal(rows, np.arange(Tn)) else x.index_select(0, rows_d.long())
         hn = ops.layernorm_nobias(xl, self._w["final_norm"], cfg.norm_eps)
+        # rows at a pitch of vocab rounded up to 8: 16-byte aligned bf16 rows for the samplers, whatever the vocabulary
+        out = torch.empty(hn.shape[0], _al8(cfg.vocab), dtype=logits_dtype, device=dev)[:, : cfg.vocab]
         if logits_dtype == torch.bfloat16 and T == torch.bfloat16:
-            return self._linear(hn, self._w["head"], out_dtype=torch.bfloat16)
-        return ops.linear_any(hn, self._w["head"], out_dtype=logits_dtype)
+            return self._linear(hn, self._w["head"], out=out)
+        return ops.linear_any(hn, self._w["head"], out=out)
 
     _trace = None      # a list: step() appends the stream after every layer (debugging / tests)
 
@@ -348,7 +351,7 @@ class LanguageModel:
             entries.append((c[0]._seq, ids[o:o + n]))
             o += n
         lg = self.step(entries, want=logits_rows, reserve_extra=reserve_extra, logits_dtype=torch.bfloat16)
-        return lg.to(torch.bfloat16) if lg.dtype != torch.bfloat16 else lg
+        return lg
 
     def decode_state(self, B: int):
         raise NotImplementedError("logits processors (penalties / logit_bias) are not built for this model")
