@@ -330,7 +330,8 @@ def test_su_rope_long_factor_regime_switches_per_call(tiny, prompt_len):
             top2 = r.topk(2).values
             assert float(top2[0] - top2[1]) < 0.06 * float(r.pow(2).mean().sqrt()), (i, toks, ref_toks)
             break
-    assert toks[0] == ref_toks[0]
+    # (the first token is covered by the loop's rule as well: on this random model the two best logits of a 4090-token prompt
+    #  can lie within the rounding of the bf16 chain, and which one wins then depends on the summation order of a build)
     # back to a short prompt afterwards: the table must have been switched back
     ids2, _, _ = _request(cfg, [], seed=77)
     f2 = np.random.default_rng(78).integers(3, 1000, 4)
