@@ -567,6 +567,12 @@ int vlm_vit_forward(void* handle, const vlm_vit_args* a, void* stream);
 int vlm_linear_any(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc, int a_f32, int w_f32,
                    int c_f32, int batch, long strideA, long strideW, long strideC, int accumulate, void* stream);
 
+/* The decode-step form (M <= 8 rows, bf16 W with 16-byte aligned rows, K % 8 == 0): 16-byte weight loads; weights whose 8
+ * activations are zero in every row are not read; skip_gate (fp32 [M][E], may be NULL): output columns [skip_col0, skip_col0 +
+ * E * ff) are E stacked experts of ff columns, a column of an expert with a zero gate in every row is written as 0 unread. */
+int vlm_linear_rows_bf16w(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc, int a_f32, int c_f32,
+                          int accumulate, const void* skip_gate, int skip_col0, int E, int ff, void* stream);
+
 /* csrc/stream_f32.hip: x is the fp32 stream [rows][D] */
 int vlm_embed_scale_f32(const void* ids, const void* table, float scale, void* x, int rows, int D, int vocab, int dtype, void* stream);
 int vlm_layernorm_nobias(const void* x, const void* w, void* out, int rows, int D, long ldo, float eps, int dtype, void* stream);

@@ -185,6 +185,7 @@ SIGNATURES = {
     "vlm_vit_set_globals": (c_int, [c_void_p, P(VitGlobals)]),
     "vlm_vit_forward": (c_int, [c_void_p, P(VitArgs), c_void_p]),
     "vlm_linear_any": (c_int, [c_void_p] * 3 + [c_int] * 3 + [C.c_long] * 3 + [c_int] * 4 + [C.c_long] * 3 + [c_int, c_void_p]),
+    "vlm_linear_rows_bf16w": (c_int, [c_void_p] * 3 + [c_int] * 3 + [C.c_long] * 3 + [c_int] * 3 + [c_void_p, c_int, c_int, c_int, c_void_p]),
     "vlm_embed_scale_f32": (c_int, [c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "vlm_layernorm_nobias": (c_int, [c_void_p] * 3 + [c_int, c_int, C.c_long, c_float, c_int, c_void_p]),
     "vlm_stream_add": (c_int, [c_void_p, c_void_p, C.c_long, c_void_p, C.c_long, c_int, c_int, c_int, c_void_p]),

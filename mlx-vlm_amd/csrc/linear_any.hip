@@ -110,6 +110,64 @@ __global__ __launch_bounds__(256) void linear_rows_kernel(const TA* __restrict__
   }
 }
 
+// the same for bf16 weights whose rows are 16-byte aligned with K a multiple of 8: every lane reads 8 weights per load
+// (16 bytes, non-temporal: a decode step reads each weight once).  Two ways to skip weights that cannot matter, both exact:
+//   * a lane whose 8 activations are zero in EVERY row does not load its 8 weights (the down projection of stacked experts:
+//     the experts no row of the step chose are exact zeros in the activations);
+//   * skip_gate != nullptr: output columns [skip_col0, skip_col0 + E * ff) belong to E stacked experts of ff columns each;
+//     a column whose expert has a zero gate in every row is written as 0 without reading its weights (the up projection).
+template <typename TA, typename TC>
+__global__ __launch_bounds__(256) void linear_rows_vec_kernel(const TA* __restrict__ A, const bf16_t* __restrict__ W, TC* __restrict__ C,
+                                                              int M, int N, int K, long lda, long ldw, long ldc, int accumulate,
+                                                              const float* __restrict__ skip_gate, int skip_col0, int E, int ff) {
+  const int n = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (n >= N) return;
+  if (skip_gate && n >= skip_col0 && n < skip_col0 + E * ff) {
+    const int e = (n - skip_col0) / ff;
+    bool any = false;
+    for (int m = 0; m < M; ++m) any |= skip_gate[(long)m * E + e] != 0.f;
+    if (!any) {                                          // (wave-uniform)
+      if (lane < M && !accumulate) st_f(C + (long)lane * ldc + n, 0.f);
+      return;
+    }
+  }
+  const bf16_t* w = W + (long)n * ldw;
+  float acc[8] = {};
+  for (int k = lane * 8; k < K; k += 512) {
+    float a[8][8];
+    bool nz = false;
+#pragma unroll
+    for (int m = 0; m < 8; ++m)
+      if (m < M) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          a[m][j] = ld_f(A + (long)m * lda + k + j);
+          nz |= a[m][j] != 0.f;
+        }
+      }
+    if (!nz) continue;
+    const uint4 wv = nt_load16(w + k);
+    const float wf[8] = {bf_lo(wv.x), bf_hi(wv.x), bf_lo(wv.y), bf_hi(wv.y), bf_lo(wv.z), bf_hi(wv.z), bf_lo(wv.w), bf_hi(wv.w)};
+#pragma unroll
+    for (int m = 0; m < 8; ++m)
+      if (m < M) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[m] = fmaf(a[m][j], wf[j], acc[m]);
+      }
+  }
+#pragma unroll
+  for (int m = 0; m < 8; ++m) {
+    if (m >= M) break;
+    float v = acc[m];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    if (lane == 0) {
+      TC* c = C + (long)m * ldc + n;
+      st_f(c, accumulate ? ld_f(c) + v : v);
+    }
+  }
+}
+
 template <typename TA, typename TW, typename TC>
 int launch(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc, int batch, long sA, long sW,
            long sC, int accumulate, hipStream_t st) {
@@ -130,6 +188,28 @@ int launch(const void* A, const void* W, void* C, int M, int N, int K, long lda,
 }
 
 }  // namespace
+
+// decode-step form with the expert-column skip (see linear_rows_vec_kernel); M <= 8, bf16 weights, K % 8 == 0
+extern "C" int vlm_linear_rows_bf16w(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc, int a_f32,
+                                     int c_f32, int accumulate, const void* skip_gate, int skip_col0, int E, int ff, void* stream) {
+  if (!A || !W || !C || M <= 0 || M > 8 || N <= 0 || K <= 0 || lda < K || ldw < K || ldc < N) return VLM_ERR_ARG;
+  if (accumulate && !c_f32) return VLM_ERR_ARG;
+  if (skip_gate && (E <= 0 || ff <= 0 || skip_col0 < 0 || skip_col0 + (long)E * ff > N)) return VLM_ERR_ARG;
+  if (K % 8 || ldw % 8 || ((uintptr_t)W & 15)) return VLM_ERR_SHAPE;
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid((N + 3) / 4);
+#define GO(TA, TC)                                                                                                              \
+  hipLaunchKernelGGL((linear_rows_vec_kernel<TA, TC>), grid, dim3(256), 0, st, (const TA*)A, (const bf16_t*)W, (TC*)C, M, N, K, lda, \
+                     ldw, ldc, accumulate, (const float*)skip_gate, skip_col0, E, ff)
+  if (a_f32) {
+    if (c_f32) GO(float, float); else GO(float, bf16_t);
+  } else {
+    if (c_f32) GO(bf16_t, float); else GO(bf16_t, bf16_t);
+  }
+#undef GO
+  VLM_CHECK_LAUNCH();
+  return VLM_OK;
+}
 
 extern "C" int vlm_linear_any(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc, int a_f32,
                               int w_f32, int c_f32, int batch, long strideA, long strideW, long strideC, int accumulate,

@@ -111,6 +111,7 @@ class LanguageModel:
         self.pool: Optional[HybridPool] = None
         self._L: List[SimpleNamespace] = []
         self._w: Dict[str, torch.Tensor] = {}
+        self._graphs: Dict[tuple, object] = {}       # captured decode steps, see _decode_rows
 
     @property
     def layers(self):
@@ -195,25 +196,37 @@ class LanguageModel:
         return [self.make_cache() for _ in range(n)]
 
     # ------------------------------------------------------------------ GEMM routing
-    def _linear(self, a, w, out=None, out_dtype=None):
+    def _linear(self, a, w, out=None, out_dtype=None, skip=None, accumulate=False):
         """a [M, K] @ w[N, K]^T: the MFMA GEMM for bf16 operands of a prompt-sized batch with 8-aligned shapes, the generic
-        kernel for everything else (fp32 mode, decode rows, odd shapes, fp32 outputs)"""
+        kernel for everything else (fp32 mode, odd shapes, fp32 outputs), and for the up-to-8 rows of a decode step over bf16
+        weights the weight-streaming form (`skip`: the expert-column skip of ops.linear_rows_bf16w)"""
         M, K = a.shape
         N = w.shape[0]
         want = out.dtype if out is not None else (out_dtype or a.dtype)
-        if (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and want == torch.bfloat16 and M > 8 and K % 8 == 0 and N % 8 == 0
+        if (not accumulate and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and want == torch.bfloat16 and M > 8 and K % 8 == 0 and N % 8 == 0
                 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and (out is None or out.stride(0) % 8 == 0)
                 and a.data_ptr() % 16 == 0 and (out is None or out.data_ptr() % 16 == 0)):
             return ops.gemm(a, w, out=out)
-        return ops.linear_any(a, w, out=out, out_dtype=out_dtype)
+        if M <= 8 and w.dtype == torch.bfloat16 and K % 8 == 0 and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0:
+            return ops.linear_rows_bf16w(a, w, out=out, out_dtype=out_dtype, accumulate=accumulate, **(skip or {}))
+        return ops.linear_any(a, w, out=out, out_dtype=out_dtype, accumulate=accumulate)
 
     # ------------------------------------------------------------------ the step
     def step(self, entries, want="last", advance: bool = True, reserve_extra: int = 0, logits_dtype=torch.float32):
         """entries: [(PagedSequence, ids)] - ids a host int array or a device int32 tensor, the NEXT tokens of that sequence.
         want: "last" (one row per entry), "all", or one list of indices (into the entry's ids) per entry.
         -> logits [wanted rows in entry order, vocab] of logits_dtype (None when nothing is wanted)."""
-        cfg, dev, T = self.config, self.device, self.dtype
-        f32 = torch.float32
+        plan = self._plan(entries, want, reserve_extra)
+        out = self._run(plan, logits_dtype)
+        if advance:
+            for s, n in zip(plan.seqs, plan.lens):
+                s.offset += n
+        return out
+
+    def _plan(self, entries, want="last", reserve_extra: int = 0, static=None):
+        """Host side of a step: pages reserved, the per-token / per-segment tables built and uploaded in ONE copy.
+        static: (int32 device buffer, ids tensor) of a captured step to refill instead of allocating."""
+        dev = self.device
         lens = [int(ids.numel() if isinstance(ids, torch.Tensor) else np.asarray(ids).size) for _, ids in entries]
         if not entries or min(lens) <= 0:
             raise ValueError("step: every entry brings at least one token")
@@ -224,9 +237,9 @@ class LanguageModel:
         for s, n in zip(seqs, lens):
             s.reserve(s.offset + n + reserve_extra)
         cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
-        if want == "last":
+        if isinstance(want, str) and want == "last":
             rows = cu[1:] - 1
-        elif want == "all":
+        elif isinstance(want, str) and want == "all":
             rows = np.arange(Tn, dtype=np.int32)
         else:
             rows = np.concatenate([cu[j] + np.asarray(w, dtype=np.int32).reshape(-1) for j, w in enumerate(want)] or [np.zeros(0, np.int32)])
@@ -235,31 +248,52 @@ class LanguageModel:
         tok_pos = np.concatenate([np.arange(s.offset, s.offset + n, dtype=np.int32) for s, n in zip(seqs, lens)])
         seg_slot = np.asarray([s.seq for s in seqs], dtype=np.int32)
         seg_pos0 = np.asarray([s.offset for s in seqs], dtype=np.int32)
-        host_ids = all(not isinstance(ids, torch.Tensor) for _, ids in entries)
+        host_ids = static is None and all(not isinstance(ids, torch.Tensor) for _, ids in entries)
         meta = [tok_seq, tok_pos, cu, seg_slot, seg_pos0, rows]
         if host_ids:
             meta.append(np.concatenate([np.asarray(ids, dtype=np.int32).reshape(-1) for _, ids in entries]))
-        md = _lib.h2d(np.concatenate(meta), dev)
-        o = 0
-        parts = []
+        host = np.concatenate(meta)
+        if static is not None:
+            md = static[0]
+            md[: host.size].copy_(_lib.h2d(host, dev))
+        else:
+            md = _lib.h2d(host, dev)
+        o, parts = 0, []
         for a in meta:
             parts.append(md[o:o + a.size])
             o += a.size
-        tok_seq_d, tok_pos_d, cu_d, slot_d, pos0_d, rows_d = parts[:6]
-        if host_ids:
+        if static is not None:
+            ids_d = static[1]
+        elif host_ids:
             ids_d = parts[6]
         else:
             ids_d = torch.cat([(ids if isinstance(ids, torch.Tensor) else _lib.h2d(np.asarray(ids, dtype=np.int32), dev))
                                .reshape(-1).to(torch.int32) for _, ids in entries])
+        return SimpleNamespace(seqs=seqs, lens=lens, nseg=nseg, Tn=Tn, rows=rows, all_rows=bool(rows.size == Tn and np.array_equal(rows, np.arange(Tn))),
+                               tok_seq=parts[0], tok_pos=parts[1], cu=parts[2], slot=parts[3], pos0=parts[4], rows_d=parts[5], ids=ids_d, md=md)
+
+    def _run(self, pl, logits_dtype=torch.float32):
+        """Device side of a step: nothing here looks at host data that changes between two steps of the same shape, so a
+        decode step can be captured once and replayed."""
+        cfg, dev, T = self.config, self.device, self.dtype
+        f32 = torch.float32
+        nseg, Tn = pl.nseg, pl.Tn
+        tok_seq_d, tok_pos_d, cu_d, slot_d, pos0_d, ids_d = pl.tok_seq, pl.tok_pos, pl.cu, pl.slot, pl.pos0, pl.ids
         pool, bt = self.pool, self.pool.block_table
         is32 = T == f32
+        few = Tn <= 8 and not is32           # decode rows over bf16 weights: weight-streaming projections with the expert skip
         x = ops.embed_scale_f32(ids_d, self._w["embed"], cfg.embedding_scale)
-        keep = [md, ids_d]
+        keep = [pl.md, ids_d]
         for i, ns in enumerate(self._L):
             h = ops.layernorm_nobias(x, ns.norm1, cfg.norm_eps)
-            proj = self._linear(h, ns.wproj)
+            gate = None
+            if ns.cfg.mlp is not None:
+                z = self._linear(h, ns.router, out_dtype=f32)
+                gate, _, _ = ops.moe_route(z, ns.top)
+                keep += [z, gate]
+            skip = dict(skip_gate=gate, skip_col0=ns.off["up"], E=ns.E, ff=ns.ff) if (few and gate is not None) else None
+            proj = self._linear(h, ns.wproj, skip=skip)
             cat = torch.zeros(Tn, ns.wout.shape[1], dtype=T, device=dev)
-            esz = proj.element_size()
             col = lambda name: proj[:, ns.off[name]:]          # noqa: E731   (2-D view: data_ptr at the column, stride(0) = pitch)
             if ns.type in ("retention", "mlstm"):
                 gated = ns.type == "mlstm"
@@ -303,39 +337,33 @@ class LanguageModel:
                 ops.linear_any(ol.view(Tn, H * R), ns.uv.view(H * Dv, R), out=cat, M=Tn, N=Dv, K=R, batch=H, stride_a=R, stride_w=Dv * R,
                                stride_c=Dv)
                 keep += [qabs, ol]
-            if ns.cfg.mlp is not None:
-                z = ops.linear_any(h, ns.router, out_dtype=f32)
-                gate, _, _ = ops.moe_route(z, ns.top)
+            if gate is not None:
                 ops.moe_relu2_gate(col("up"), gate, ns.E, ns.ff, ns.sff, cat[:, ns.koff["ff"]:])
-                keep += [z, gate]
             if T == torch.bfloat16 and Tn > 8:
                 y = self._linear(cat, ns.wout)
                 ops.stream_add_(x, y)
                 keep.append(y)
+            elif few:
+                self._linear(cat, ns.wout, out=x, accumulate=True)      # (unchosen experts: zero activations, weights not read)
             else:
                 ops.linear_any(cat, ns.wout, out=x, accumulate=True)
             if cfg.side_dim:
-                sg = ops.linear_any(x, ns.side_gate, out_dtype=T)
+                sg = self._linear(x, ns.side_gate, out_dtype=T)
                 gg = ops.gelu_tanh_gate_rows(sg, self._w["side_embed"], ids_d, i * cfg.side_dim)
-                y2 = ops.linear_any(gg, ns.side_proj)
+                y2 = self._linear(gg, ns.side_proj)
                 ops.unit_rms_add_(x, y2, ns.side_norm, cfg.norm_eps)
                 keep += [sg, gg, y2]
             keep += [h, proj, cat]
             if self._trace is not None:
                 self._trace.append(x.clone())
-        if advance:
-            for s, n in zip(seqs, lens):
-                s.offset += n
         self._keep = keep
-        if rows.size == 0:
+        if pl.rows.size == 0:
             return None
-        xl = x if rows.size == Tn and np.array_equal(rows, np.arange(Tn)) else x.index_select(0, rows_d.long())
+        xl = x if pl.all_rows else x.index_select(0, pl.rows_d.long())
         hn = ops.layernorm_nobias(xl, self._w["final_norm"], cfg.norm_eps)
         # rows at a pitch of vocab rounded up to 8: 16-byte aligned bf16 rows for the samplers, whatever the vocabulary
         out = torch.empty(hn.shape[0], _al8(cfg.vocab), dtype=logits_dtype, device=dev)[:, : cfg.vocab]
-        if logits_dtype == torch.bfloat16 and T == torch.bfloat16:
-            return self._linear(hn, self._w["head"], out=out)
-        return ops.linear_any(hn, self._w["head"], out=out)
+        return self._linear(hn, self._w["head"], out=out)
 
     _trace = None      # a list: step() appends the stream after every layer (debugging / tests)
 
@@ -381,14 +409,46 @@ class LanguageModel:
         if lp is not None:
             st.logprobs[:n].copy_(lp)
 
+    def _decode_rows(self, st: DecodeRows, seqs, sampler_args: dict, with_logprobs: bool, use_graph: bool, advance: bool):
+        """One decode step of rows 0..n-1 of st (one token each, fed from st.tok): forward, sampling on the device, the sampled
+        token written back as the next input.  With use_graph the launch sequence of a (state, row count, sampler) is captured
+        into a HIP graph the second time it runs and replayed from then on: the host then only reserves pages and refills the
+        small table of (sequence slot, position) per row - a step is ~100 launches, which the host cannot issue as fast as the
+        GPU runs them."""
+        n = len(seqs)
+        entries = [(s, st.tok[r:r + 1]) for r, s in enumerate(seqs)]
+        key = (id(st), n, bool(with_logprobs), tuple(sorted(sampler_args.items())))
+        ent = self._graphs.get(key) if use_graph else None
+        if ent is None:
+            self._rows_step(st, seqs, advance=False)
+            self._sample_rows(st, n, sampler_args, with_logprobs)
+            self.decode_advance_rows(st, n)
+            if use_graph:
+                self._graphs[key] = "seen"           # the first run loads the kernels; the second one is captured
+        else:
+            if ent == "seen":
+                meta = torch.zeros(6 * n + 1, dtype=torch.int32, device=self.device)
+                pl = self._plan(entries, "last", static=(meta, st.tok[:n]))
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    lg = self._run(pl, torch.bfloat16)
+                    st.logits[:n].copy_(lg)
+                    self._sample_rows(st, n, sampler_args, with_logprobs)
+                    self.decode_advance_rows(st, n)
+                ent = self._graphs[key] = (g, meta, st, self._keep, lg)
+            else:
+                self._plan(entries, "last", static=(ent[1], st.tok[:n]))
+            ent[0].replay()
+        if advance:
+            for s in seqs:
+                s.offset += 1
+
     def decode_run(self, st: DecodeRows, n_steps: int, sampler_args: dict, use_graph: bool = True, penalties=None):
         """n_steps decode steps of st's rows: step, sample on the device, feed the sampled token back"""
         if penalties:
             raise NotImplementedError("logits processors are not built for this model")
         for _ in range(n_steps):
-            self._rows_step(st, st.seqs, advance=True)
-            self._sample_rows(st, len(st.seqs), sampler_args)
-            self.decode_advance_rows(st, len(st.seqs))
+            self._decode_rows(st, st.seqs, sampler_args, True, use_graph, advance=True)
 
     def decode_step_rows(self, st: DecodeRows, B: int, block_table, sampler_args: dict, use_graph: bool = True,
                          with_logprobs: bool = True, row_penalties: bool = False, q8: bool = False):
@@ -396,10 +456,7 @@ class LanguageModel:
         past them are idle and are not run.  The scheduler advances the sequences' offsets itself."""
         if row_penalties or q8:
             raise NotImplementedError("per-request logits processors / quantized caches are not built for this model")
-        n = len(st.row_seqs)
-        self._rows_step(st, st.row_seqs, advance=False)
-        self._sample_rows(st, n, sampler_args, with_logprobs)
-        self.decode_advance_rows(st, n)
+        self._decode_rows(st, st.row_seqs, sampler_args, with_logprobs, use_graph, advance=False)
 
     def decode_forward_rows(self, st: DecodeRows, B: int, block_table, q8: bool = False):
         self._rows_step(st, st.row_seqs, advance=False)

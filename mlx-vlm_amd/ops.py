@@ -575,6 +575,19 @@ def linear_any(a, w, out=None, out_dtype=None, accumulate=False, batch=1, stride
     return out
 
 
+def linear_rows_bf16w(a, w, out=None, out_dtype=None, accumulate=False, skip_gate=None, skip_col0=0, E=0, ff=0):
+    """the decode-step form of linear_any (up to 8 rows, bf16 weights, K % 8 == 0): see vlm_linear_rows_bf16w"""
+    _dev(a, w, out, skip_gate)
+    M, K = a.shape
+    N = w.shape[0]
+    if out is None:
+        out = torch.empty(M, N, dtype=out_dtype or a.dtype, device=a.device)
+    check(_lib.lib().vlm_linear_rows_bf16w(_p(a), _p(w), _p(out), M, N, K, a.stride(0), w.stride(0), out.stride(0), _f32(a), _f32(out),
+                                           int(bool(accumulate)), _p(skip_gate), int(skip_col0), int(E), int(ff), _stream()),
+          "linear_rows_bf16w")
+    return out
+
+
 def embed_scale_f32(ids, table, scale, out=None):
     """x [T, D] fp32 = table[ids] * scale"""
     _dev(ids, table, out)

@@ -379,3 +379,36 @@ def test_trace_session_replays_mixed_steps(tmp_path):
     lg = s.step([("b", b[29:].tolist(), [0]), ("a", a[99:].tolist(), [0])], end=["a", "b"])
     assert H.rel_rms(lg, torch.stack([wb[29], wa[99]])) < TOL["float32"]
     assert model.language_model.pool.free_pages == 4
+
+
+def test_captured_decode_steps_equal_eager_ones(tmp_path):
+    """a captured decode step is replayed many times, with eager work (another request's prompt, a release, synchronisations)
+    between the replays; every replay's logits and token must equal the eager step's"""
+    from mlx_vlm_amd.sample_utils import make_sampler
+
+    cfg = H.config(H.MIXED)
+    W = H.weights(cfg, seed=71)
+    lm = _load(tmp_path, cfg, W, "bfloat16", tokens=2048, seqs=6).language_model
+    sargs = make_sampler().engine_args()
+    prompts = [_ids(n, cfg["vocab"], 80 + n) for n in (40, 7, 66)]
+
+    def run(use_graph):
+        caches = lm.make_cache_batch(3)
+        lg = lm.prefill(torch.cat([torch.as_tensor(p) for p in prompts]).cuda().reshape(-1, 1), None, caches, [len(p) for p in prompts])
+        st = lm.decode_begin(caches, lg.argmax(-1), np.zeros((3, 1)), max_new_tokens=80)
+        out = []
+        for i in range(70):                                          # crosses a page border in every row
+            lm.decode_run(st, 1, sargs, use_graph=use_graph)
+            out.append((st.tok.cpu().clone(), st.logits.float().cpu().clone()))
+            if i % 9 == 4:                                           # eager work between replays
+                other = lm.make_cache()
+                lm.step([(other[0]._seq, _ids(30 + i, cfg["vocab"], i))])
+                torch.cuda.synchronize()
+                other[0]._seq.release()
+        for c in caches:
+            c[0]._seq.release()
+        return out
+    eager, graph = run(False), run(True)
+    assert any(isinstance(v, tuple) for v in lm._graphs.values())            # a graph was captured and used
+    for i, ((t0, l0), (t1, l1)) in enumerate(zip(eager, graph)):
+        assert torch.equal(t0, t1) and torch.equal(l0, l1), i
