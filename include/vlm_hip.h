@@ -619,6 +619,11 @@ int vlm_rope_pairs_rows(const void* q, long ldq, long head_stride, int H, int Dr
                         long ldo, long out_head_stride, int rows, int dtype, void* stream);
 int vlm_latent_attn(const void* q, const void* pool, const void* tok_seq, const void* tok_pos, const void* block_table, int max_pages,
                     int H, int R, int Dr, float scale, const void* gate, long ldgate, void* out, int rows, int dtype, void* stream);
+/* the prompt form: query blocks (first token, count <= 16, all of one sequence and consecutive) x heads, key tiles through LDS;
+ * R <= 512.  Same results as vlm_latent_attn up to summation order. */
+int vlm_latent_attn_blocks(const void* q, const void* pool, const void* qb_start, const void* qb_count, int nblocks, const void* tok_seq,
+                           const void* tok_pos, const void* block_table, int max_pages, int H, int R, int Dr, float scale,
+                           const void* gate, long ldgate, void* out, int dtype, void* stream);
 
 /* csrc/moe.hip */
 int vlm_moe_route(const void* logits, int T, int E, int top, void* gate, void* idx, void* wgt, void* stream);

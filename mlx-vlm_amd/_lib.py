@@ -198,6 +198,8 @@ SIGNATURES = {
     "vlm_rope_pairs_rows": (c_int, [c_void_p, C.c_long, C.c_long, c_int, c_int, c_void_p, c_void_p, c_void_p, C.c_long, C.c_long,
                                     c_int, c_int, c_void_p]),
     "vlm_latent_attn": (c_int, [c_void_p] * 5 + [c_int] * 4 + [c_float, c_void_p, C.c_long, c_void_p, c_int, c_int, c_void_p]),
+    "vlm_latent_attn_blocks": (c_int, [c_void_p] * 4 + [c_int] + [c_void_p] * 3 + [c_int] * 4 + [c_float, c_void_p, C.c_long, c_void_p,
+                                       c_int, c_void_p]),
     "vlm_moe_route": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "vlm_moe_relu2_gate": (c_int, [c_void_p, C.c_long, c_void_p, c_int, c_int, c_int, c_void_p, C.c_long, c_int, c_int, c_void_p]),
 }

@@ -151,6 +151,153 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(const float* __restric
   }
 }
 
+// Prompt form: workgroup = (block of up to QB consecutive query tokens of one sequence, head).  Key tiles of KT cached rows are
+// staged through LDS once for all queries of the block; tile j covers keys [KT j, KT j + KT) counted from the sequence's first
+// token, and every query runs the same per-tile update in the same order whatever block it sits in (a tile that holds no
+// visible key for a query leaves its running maximum, sum and accumulator untouched bit for bit), so a token's result does
+// not depend on how the prompt was cut or batched.
+constexpr int QB = 16, KT = 16;
+
+__device__ __forceinline__ void load8(const bf16_t* p, float* f) {
+  const uint4 v = *reinterpret_cast<const uint4*>(p);
+  f[0] = bf_lo(v.x); f[1] = bf_hi(v.x); f[2] = bf_lo(v.y); f[3] = bf_hi(v.y);
+  f[4] = bf_lo(v.z); f[5] = bf_hi(v.z); f[6] = bf_lo(v.w); f[7] = bf_hi(v.w);
+}
+__device__ __forceinline__ void load8(const float* p, float* f) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+}
+
+// DP: the row pitch of q and k in LDS, Dk rounded up to 8 (+ 4 for the key rows: 16-byte aligned rows whose 16 starts
+// spread over the banks); the pad columns hold zeros, so the 4-wide dot product runs over them
+template <typename T, int NACC>
+__global__ __launch_bounds__(256) void latent_attn_block_kernel(const float* __restrict__ q, const T* __restrict__ pool,
+                                                                const int* __restrict__ qb_start, const int* __restrict__ qb_count,
+                                                                const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+                                                                const int* __restrict__ block_table, int max_pages, int H, int R,
+                                                                int Dr, float scale, const T* __restrict__ gate, long ldgate,
+                                                                float* __restrict__ out) {
+  extern __shared__ float smem[];
+  const int Dk = R + Dr, DP = (Dk + 7) & ~7, KP = DP + 4;
+  float* qs = smem;                         // [QB][DP]
+  float* ks = qs + QB * DP;                 // [KT][KP]
+  float* ps = ks + KT * KP;                 // [KT][QB]   (key-major: the weighted sum reads the 16 weights of a key as 4 x float4)
+  float* mrun = ps + QB * KT;               // [QB]
+  float* lrun = mrun + QB;                  // [QB]
+  float* alph = lrun + QB;                  // [QB]
+  const int t0 = qb_start[blockIdx.x], nq = qb_count[blockIdx.x];
+  const int h = blockIdx.y, tid = threadIdx.x;
+  const int* bt = block_table + (long)tok_seq[t0] * max_pages;
+  const int pos0 = tok_pos[t0];             // positions of the block's queries: pos0 .. pos0 + nq - 1
+  const int r16 = tid >> 4, l16 = tid & 15; // (row of a 16-row tile, lane within the row's 16 lanes)
+  for (int d = l16; d < DP; d += 16) qs[r16 * DP + d] = (r16 < nq && d < Dk) ? q[((long)(t0 + r16) * H + h) * Dk + d] : 0.f;
+  if (tid < QB) {
+    mrun[tid] = -INFINITY;
+    lrun[tid] = 0.f;
+  }
+  float acc[QB][NACC];
+#pragma unroll
+  for (int a = 0; a < QB; ++a)
+#pragma unroll
+    for (int b = 0; b < NACC; ++b) acc[a][b] = 0.f;
+  const int nkeys = pos0 + nq;              // the last query sees keys 0 .. pos0 + nq - 1
+  const bool vec = (Dk & 7) == 0;           // rows of the pool are 16-byte aligned and a whole number of 8-element groups
+  for (int j0 = 0; j0 < nkeys; j0 += KT) {
+    __syncthreads();                        // (qs / state initialised; the previous tile's ks and ps are no longer read)
+    {
+      const int key = j0 + r16;
+      float* dst = ks + r16 * KP;
+      if (key < nkeys) {
+        const T* src = pool + ((long)bt[key / PAGE] * PAGE + key % PAGE) * Dk;
+        if (vec) {
+          for (int d = l16 * 8; d < Dk; d += 128) {
+            float f[8];
+            load8(src + d, f);
+            *reinterpret_cast<float4*>(dst + d) = make_float4(f[0], f[1], f[2], f[3]);
+            *reinterpret_cast<float4*>(dst + d + 4) = make_float4(f[4], f[5], f[6], f[7]);
+          }
+        } else {
+          for (int d = l16; d < DP; d += 16) dst[d] = d < Dk ? ld_f(src + d) : 0.f;
+        }
+      } else {
+        for (int d = l16; d < DP; d += 16) dst[d] = 0.f;
+      }
+    }
+    __syncthreads();
+    {
+      // one (query r16, key l16) pair per lane, four dimensions per LDS read, ascending - a fixed order per pair
+      const float4* qr = reinterpret_cast<const float4*>(qs + r16 * DP);
+      const float4* kr = reinterpret_cast<const float4*>(ks + l16 * KP);
+      float d = 0.f;
+      for (int i = 0; i < DP / 4; ++i) {
+        const float4 a = qr[i], b = kr[i];
+        d = fmaf(a.x, b.x, d);
+        d = fmaf(a.y, b.y, d);
+        d = fmaf(a.z, b.z, d);
+        d = fmaf(a.w, b.w, d);
+      }
+      const bool seen = r16 < nq && j0 + l16 <= pos0 + r16;
+      ps[l16 * QB + r16] = seen ? d * scale : -INFINITY;
+    }
+    __syncthreads();
+    if (tid < QB) {                         // per query: running maximum, tile weights, running sum (fixed order over the tile)
+      float sc[KT];
+#pragma unroll
+      for (int k = 0; k < KT; ++k) sc[k] = ps[k * QB + tid];
+      float mt = sc[0];
+#pragma unroll
+      for (int k = 1; k < KT; ++k) mt = fmaxf(mt, sc[k]);
+      const float m_old = mrun[tid], m_new = fmaxf(m_old, mt);
+      float sum = 0.f;
+#pragma unroll
+      for (int k = 0; k < KT; ++k) {
+        const float pv = sc[k] == -INFINITY ? 0.f : expf(sc[k] - m_new);
+        ps[k * QB + tid] = pv;
+        sum += pv;
+      }
+      const float al = m_new == -INFINITY || m_old == m_new ? 1.f : expf(m_old - m_new);
+      alph[tid] = al;
+      lrun[tid] = lrun[tid] * al + sum;
+      mrun[tid] = m_new;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int a = 0; a < QB; ++a) {
+      const float al = alph[a];
+#pragma unroll
+      for (int b = 0; b < NACC; ++b) acc[a][b] *= al;
+    }
+#pragma unroll 2
+    for (int k = 0; k < KT; ++k) {
+      float c[NACC];
+#pragma unroll
+      for (int b = 0; b < NACC; ++b) c[b] = tid + 256 * b < R ? ks[k * KP + tid + 256 * b] : 0.f;
+      const float4* pk = reinterpret_cast<const float4*>(ps + k * QB);
+#pragma unroll
+      for (int a4 = 0; a4 < QB / 4; ++a4) {
+        const float4 pv = pk[a4];
+#pragma unroll
+        for (int b = 0; b < NACC; ++b) {
+          acc[4 * a4 + 0][b] = fmaf(pv.x, c[b], acc[4 * a4 + 0][b]);
+          acc[4 * a4 + 1][b] = fmaf(pv.y, c[b], acc[4 * a4 + 1][b]);
+          acc[4 * a4 + 2][b] = fmaf(pv.z, c[b], acc[4 * a4 + 2][b]);
+          acc[4 * a4 + 3][b] = fmaf(pv.w, c[b], acc[4 * a4 + 3][b]);
+        }
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int a = 0; a < QB; ++a) {
+    if (a >= nq) break;
+    float gsc = 1.f / lrun[a];
+    if (gate) gsc *= 1.f / (1.f + expf(-ld_f(gate + (long)(t0 + a) * ldgate + h)));
+#pragma unroll
+    for (int b = 0; b < NACC; ++b)
+      if (tid + 256 * b < R) out[((long)(t0 + a) * H + h) * R + tid + 256 * b] = acc[a][b] * gsc;
+  }
+}
+
 }  // namespace
 
 extern "C" int vlm_latent_kv_write(const void* d, long ldd, const void* w, int R, int Dr, const void* inv_freq, const void* tok_seq,
@@ -208,6 +355,41 @@ extern "C" int vlm_latent_attn(const void* q, const void* pool, const void* tok_
     if (nacc == 1) GO(float, 1); else if (nacc == 2) GO(float, 2); else GO(float, 4);
   } else {
     if (nacc == 1) GO(bf16_t, 1); else if (nacc == 2) GO(bf16_t, 2); else GO(bf16_t, 4);
+  }
+#undef GO
+  VLM_CHECK_LAUNCH();
+  return VLM_OK;
+}
+
+extern "C" int vlm_latent_attn_blocks(const void* q, const void* pool, const void* qb_start, const void* qb_count, int nblocks,
+                                      const void* tok_seq, const void* tok_pos, const void* block_table, int max_pages, int H, int R,
+                                      int Dr, float scale, const void* gate, long ldgate, void* out, int dtype, void* stream) {
+  if (!q || !pool || !qb_start || !qb_count || !tok_seq || !tok_pos || !block_table || !out || H <= 0 || R <= 0 || Dr < 0 ||
+      max_pages <= 0 || nblocks < 0 || (gate && ldgate < H))
+    return VLM_ERR_ARG;
+  if (nblocks == 0) return VLM_OK;
+  const int Dk = R + Dr;
+  const int DP = (Dk + 7) & ~7;
+  const size_t lds = ((size_t)QB * DP + (size_t)KT * (DP + 4) + QB * KT + 3 * QB) * sizeof(float);
+  if (R > 512 || H > 65535 || lds > 150 * 1024) return VLM_ERR_SHAPE;
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid(nblocks, H);
+#define GO(T, N)                                                                                                                   \
+  do {                                                                                                                             \
+    if (lds > 48 * 1024) {                                                                                                         \
+      hipError_t e = hipFuncSetAttribute((const void*)latent_attn_block_kernel<T, N>, hipFuncAttributeMaxDynamicSharedMemorySize,  \
+                                         (int)lds);                                                                                \
+      if (e != hipSuccess) return VLM_ERR_HIP + (int)e;                                                                            \
+    }                                                                                                                              \
+    hipLaunchKernelGGL((latent_attn_block_kernel<T, N>), grid, dim3(256), lds, st, (const float*)q, (const T*)pool,                \
+                       (const int*)qb_start, (const int*)qb_count, (const int*)tok_seq, (const int*)tok_pos,                       \
+                       (const int*)block_table, max_pages, H, R, Dr, scale, (const T*)gate, ldgate, (float*)out);                  \
+  } while (0)
+  const int nacc = (R + 255) / 256;
+  if (dtype) {
+    if (nacc == 1) GO(float, 1); else GO(float, 2);
+  } else {
+    if (nacc == 1) GO(bf16_t, 1); else GO(bf16_t, 2);
   }
 #undef GO
   VLM_CHECK_LAUNCH();

@@ -149,23 +149,37 @@ __global__ __launch_bounds__(1024) void linear_recurrence_kernel(vlm_recurrence_
   }
 }
 
-// the running maximum m_t per (token, head) for the finish pass, and the slot's maximum moved to the end of the segment:
-// the same scan as above, one lane per (segment, head)
+// the running maximum m_t per (token, head) for the finish pass, and the slot's maximum moved to the end of the segment: one
+// wave per (segment, head).  64 tokens at a time: every lane evaluates the gates of its token (the transcendental part, in
+// parallel), then the scan itself - a maximum and an add per token - walks the 64 lanes in order, the same sequence of
+// operations as a token-by-token loop.
 template <typename T>
-__global__ void gate_max_kernel(vlm_recurrence_args p, int nseg) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= nseg * p.H) return;
+__global__ __launch_bounds__(64) void gate_max_kernel(vlm_recurrence_args p, int nseg) {
+  const int i = blockIdx.x, lane = threadIdx.x;
   const int seg = i / p.H, h = i % p.H;
   float* ms = p.mstate + (long)p.seg_slot[seg] * p.H + h;
   float m = p.seg_pos0[seg] > 0 ? *ms : 0.f;
-  p.mprev[i] = m;
-  for (int tok = p.seg_start[seg]; tok < p.seg_start[seg + 1]; ++tok) {
-    const float iv = ld_f((const T*)p.ipre + (long)tok * p.ldi + h) + ld_f((const T*)p.ib + h);
-    const float fv = ld_f((const T*)p.fpre + (long)tok * p.ldf + h) + ld_f((const T*)p.fb + h);
-    m = fmaxf(logsigmoid_f(p.cap * tanhf(fv / p.cap)) + m, p.cap * tanhf(iv / p.cap));
-    p.mtok[(long)tok * p.H + h] = m;
+  if (lane == 0) p.mprev[i] = m;
+  const int t_end = p.seg_start[seg + 1];
+  for (int t0 = p.seg_start[seg]; t0 < t_end; t0 += 64) {
+    const int tok = t0 + lane;
+    float ig = 0.f, fg = 0.f;
+    if (tok < t_end) {
+      const float iv = ld_f((const T*)p.ipre + (long)tok * p.ldi + h) + ld_f((const T*)p.ib + h);
+      const float fv = ld_f((const T*)p.fpre + (long)tok * p.ldf + h) + ld_f((const T*)p.fb + h);
+      ig = p.cap * tanhf(iv / p.cap);
+      fg = logsigmoid_f(p.cap * tanhf(fv / p.cap));
+    }
+    const int nb = min(64, t_end - t0);
+    float mine = 0.f;
+    for (int t = 0; t < nb; ++t) {          // (t is wave-uniform: a broadcast read of lane t)
+      const float it = __shfl(ig, t), ft = __shfl(fg, t);
+      m = fmaxf(ft + m, it);
+      if (lane == t) mine = m;
+    }
+    if (tok < t_end) p.mtok[(long)tok * p.H + h] = mine;
   }
-  *ms = m;
+  if (lane == 0) *ms = m;
 }
 
 template <typename T, bool GATED>
@@ -207,7 +221,7 @@ int run(const vlm_recurrence_args& a, int nseg, int ntok, hipStream_t st) {
   dim3 grid(nseg, a.H, (C + CT - 1) / CT), block(P * CT);
   if (gated) {
     // the per-token maxima first: the scan kernel overwrites the slot's running maximum
-    hipLaunchKernelGGL(gate_max_kernel<T>, dim3((nseg * a.H + 63) / 64), dim3(64), 0, st, a, nseg);
+    hipLaunchKernelGGL(gate_max_kernel<T>, dim3(nseg * a.H), dim3(64), 0, st, a, nseg);
     VLM_CHECK_LAUNCH();
     hipLaunchKernelGGL((linear_recurrence_kernel<T, true>), grid, block, lds(TB), st, a, P, TB);
   } else {

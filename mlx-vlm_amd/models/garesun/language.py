@@ -249,7 +249,10 @@ class LanguageModel:
         seg_slot = np.asarray([s.seq for s in seqs], dtype=np.int32)
         seg_pos0 = np.asarray([s.offset for s in seqs], dtype=np.int32)
         host_ids = static is None and all(not isinstance(ids, torch.Tensor) for _, ids in entries)
-        meta = [tok_seq, tok_pos, cu, seg_slot, seg_pos0, rows]
+        # query blocks of the prompt-form attention: up to 16 consecutive tokens of one segment
+        qb = [(cu[j] + o, min(16, n - o)) for j, n in enumerate(lens) for o in range(0, n, 16)]
+        qb_start, qb_count = np.asarray([b[0] for b in qb], dtype=np.int32), np.asarray([b[1] for b in qb], dtype=np.int32)
+        meta = [tok_seq, tok_pos, cu, seg_slot, seg_pos0, rows, qb_start, qb_count]
         if host_ids:
             meta.append(np.concatenate([np.asarray(ids, dtype=np.int32).reshape(-1) for _, ids in entries]))
         host = np.concatenate(meta)
@@ -265,12 +268,13 @@ class LanguageModel:
         if static is not None:
             ids_d = static[1]
         elif host_ids:
-            ids_d = parts[6]
+            ids_d = parts[8]
         else:
             ids_d = torch.cat([(ids if isinstance(ids, torch.Tensor) else _lib.h2d(np.asarray(ids, dtype=np.int32), dev))
                                .reshape(-1).to(torch.int32) for _, ids in entries])
         return SimpleNamespace(seqs=seqs, lens=lens, nseg=nseg, Tn=Tn, rows=rows, all_rows=bool(rows.size == Tn and np.array_equal(rows, np.arange(Tn))),
-                               tok_seq=parts[0], tok_pos=parts[1], cu=parts[2], slot=parts[3], pos0=parts[4], rows_d=parts[5], ids=ids_d, md=md)
+                               tok_seq=parts[0], tok_pos=parts[1], cu=parts[2], slot=parts[3], pos0=parts[4], rows_d=parts[5], qb_start=parts[6],
+                               qb_count=parts[7], ids=ids_d, md=md)
 
     def _run(self, pl, logits_dtype=torch.float32):
         """Device side of a step: nothing here looks at host data that changes between two steps of the same shape, so a
@@ -332,8 +336,14 @@ class LanguageModel:
                                stride_c=R + Dr)
                 if Dr:
                     ops.rope_pairs_rows(proj[:, ns.off["q"] + D:], D + Dr, H, Dr, ns.inv_freq, tok_pos_d, qabs[:, R:], R + Dr)
-                ol = ops.latent_attn(qabs.view(Tn, H, R + Dr), pool.rows[ns.src], tok_seq_d, tok_pos_d, bt, H, R, Dr, ns.scale,
-                                     gate=col("g"))
+                # prompt form (key tiles shared by a block of queries) wherever a step brings more than decode rows, and always
+                # in float32 serving - one kernel there, so that a token's bits do not depend on the schedule
+                if (is32 or Tn > 8) and R <= 512 and (32 * _al8(R + Dr) + 512) * 4 <= 150 * 1024:
+                    ol = ops.latent_attn_blocks(qabs.view(Tn, H, R + Dr), pool.rows[ns.src], pl.qb_start, pl.qb_count, tok_seq_d, tok_pos_d,
+                                                bt, H, R, Dr, ns.scale, gate=col("g"))
+                else:
+                    ol = ops.latent_attn(qabs.view(Tn, H, R + Dr), pool.rows[ns.src], tok_seq_d, tok_pos_d, bt, H, R, Dr, ns.scale,
+                                         gate=col("g"))
                 ops.linear_any(ol.view(Tn, H * R), ns.uv.view(H * Dv, R), out=cat, M=Tn, N=Dv, K=R, batch=H, stride_a=R, stride_w=Dv * R,
                                stride_c=Dv)
                 keep += [qabs, ol]
@@ -427,7 +437,7 @@ class LanguageModel:
                 self._graphs[key] = "seen"           # the first run loads the kernels; the second one is captured
         else:
             if ent == "seen":
-                meta = torch.zeros(6 * n + 1, dtype=torch.int32, device=self.device)
+                meta = torch.zeros(8 * n + 1, dtype=torch.int32, device=self.device)
                 pl = self._plan(entries, "last", static=(meta, st.tok[:n]))
                 g = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(g):

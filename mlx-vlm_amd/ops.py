@@ -669,6 +669,20 @@ def latent_attn(q, pool, tok_seq, tok_pos, block_table, H, R, Dr, scale, gate=No
     return out
 
 
+def latent_attn_blocks(q, pool, qb_start, qb_count, tok_seq, tok_pos, block_table, H, R, Dr, scale, gate=None, out=None):
+    """latent_attn over query blocks (qb_start / qb_count int32 [n]: first token and number of consecutive tokens of one
+    sequence, at most 16): the prompt form, key tiles staged once per block"""
+    _dev(q, pool, qb_start, qb_count, tok_seq, tok_pos, block_table, gate, out)
+    T = q.shape[0]
+    if out is None:
+        out = torch.empty(T, H, R, dtype=torch.float32, device=q.device)
+    check(_lib.lib().vlm_latent_attn_blocks(_p(q), _p(pool), _p(qb_start), _p(qb_count), qb_start.numel(), _p(tok_seq), _p(tok_pos),
+                                            _p(block_table), block_table.shape[1], int(H), int(R), int(Dr), float(scale), _p(gate),
+                                            gate.stride(0) if gate is not None else 0, _p(out), _f32(pool), _stream()),
+          "latent_attn_blocks")
+    return out
+
+
 def moe_route(logits, top):
     """fp32 logits [T, E] -> (dense gate table fp32 [T, E], chosen indices int32 [T, top], their weights fp32 [T, top])"""
     _dev(logits)

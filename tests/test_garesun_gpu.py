@@ -412,3 +412,35 @@ def test_captured_decode_steps_equal_eager_ones(tmp_path):
     assert any(isinstance(v, tuple) for v in lm._graphs.values())            # a graph was captured and used
     for i, ((t0, l0), (t1, l1)) in enumerate(zip(eager, graph)):
         assert torch.equal(t0, t1) and torch.equal(l0, l1), i
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_latent_attention_prompt_form_equals_row_form(dtype):
+    """the two attention kernels (query blocks through LDS / one row per workgroup) against a dense softmax, ragged batch:
+    two sequences at different offsets on scattered pages, blocks that end inside a tile"""
+    from mlx_vlm_amd import ops
+    from mlx_vlm_amd.models.cache import PAGE
+
+    R, Dr, Hh = 40, 8, 3
+    g = torch.Generator().manual_seed(9)
+    lens, offs = [37, 5], [150, 0]                   # sequence 0: 37 new tokens after 150 cached ones; sequence 1: 5 from the start
+    bt = torch.zeros(3, 8, dtype=torch.int32)
+    bt[1, :3] = torch.tensor([5, 2, 7])
+    bt[2, :1] = torch.tensor([4])
+    pool = (torch.randn(8, PAGE, R + Dr, generator=g) * 0.5).to(dtype)
+    tok_seq = torch.tensor([1] * 37 + [2] * 5, dtype=torch.int32)
+    tok_pos = torch.tensor(list(range(150, 187)) + list(range(5)), dtype=torch.int32)
+    q = torch.randn(42, Hh, R + Dr, generator=g)
+    gate = torch.randn(42, Hh, generator=g).to(dtype)
+    qb_start = torch.tensor([0, 16, 32, 37], dtype=torch.int32)
+    qb_count = torch.tensor([16, 16, 5, 5], dtype=torch.int32)
+    a = ops.latent_attn(q.cuda(), pool.cuda(), tok_seq.cuda(), tok_pos.cuda(), bt.cuda(), Hh, R, Dr, 0.3, gate=gate.cuda()).cpu()
+    b = ops.latent_attn_blocks(q.cuda(), pool.cuda(), qb_start.cuda(), qb_count.cuda(), tok_seq.cuda(), tok_pos.cuda(), bt.cuda(), Hh, R, Dr,
+                               0.3, gate=gate.cuda()).cpu()
+    want = torch.zeros(42, Hh, R, dtype=torch.float64)
+    for t in range(42):
+        sq, pos = int(tok_seq[t]), int(tok_pos[t])
+        rows = torch.stack([pool[bt[sq, j // PAGE], j % PAGE] for j in range(pos + 1)]).double()
+        w = torch.softmax(torch.einsum("hd,jd->hj", q[t].double(), rows) * 0.3, -1)
+        want[t] = torch.einsum("hj,jr->hr", w, rows[:, :R]) * torch.sigmoid(gate[t].double())[:, None]
+    assert (a.double() - want).abs().max() < 2e-5 and (b.double() - want).abs().max() < 2e-5
