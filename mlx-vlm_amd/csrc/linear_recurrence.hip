@@ -36,7 +36,7 @@ __device__ __forceinline__ float logsigmoid_f(float x) { return fminf(x, 0.f) - 
 
 template <typename T, bool GATED>
 __global__ __launch_bounds__(1024) void linear_recurrence_kernel(vlm_recurrence_args p, int P, int TB) {
-  extern __shared__ float smem[];
+  extern __shared__ __align__(16) float smem[];
   const int seg = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * CT;
   const int D = p.D, Dv = p.Dv, C = Dv + (GATED ? 1 : 0), DP = P * DR;
   const int tid = threadIdx.x, nthr = blockDim.x;
@@ -121,13 +121,21 @@ __global__ __launch_bounds__(1024) void linear_recurrence_kernel(vlm_recurrence_
     for (int t = 0; t < nb; ++t) {
       const float a = GATED ? ab[t * 4 + 0] : dec, b = GATED ? ab[t * 4 + 1] : 1.f;
       const float bv = b * vs[t * CT + (tid % CT)];
-      const float* kr = ks + t * DP + row0;
-      const float* qr = qs + t * DP + row0;
+      // (k and q of the token are the same for every lane of the wave: 16-byte broadcast reads, rows ascending)
+      const float4* kr = reinterpret_cast<const float4*>(ks + t * DP + row0);
+      const float4* qr = reinterpret_cast<const float4*>(qs + t * DP + row0);
       float acc = 0.f;
 #pragma unroll
-      for (int r = 0; r < DR; ++r) {
-        s[r] = fmaf(a, s[r], kr[r] * bv);
-        acc = fmaf(s[r], qr[r], acc);
+      for (int r = 0; r < DR / 4; ++r) {
+        const float4 kk = kr[r], qq = qr[r];
+        s[4 * r + 0] = fmaf(a, s[4 * r + 0], kk.x * bv);
+        acc = fmaf(s[4 * r + 0], qq.x, acc);
+        s[4 * r + 1] = fmaf(a, s[4 * r + 1], kk.y * bv);
+        acc = fmaf(s[4 * r + 1], qq.y, acc);
+        s[4 * r + 2] = fmaf(a, s[4 * r + 2], kk.z * bv);
+        acc = fmaf(s[4 * r + 2], qq.z, acc);
+        s[4 * r + 3] = fmaf(a, s[4 * r + 3], kk.w * bv);
+        acc = fmaf(s[4 * r + 3], qq.w, acc);
       }
       po[(t * P + part) * CT + (tid % CT)] = acc;
     }
