@@ -20,11 +20,11 @@ def garesun_cfg(s):
     H, hd, W = s["heads"], s["hd"], s["width"]
     ff = s["inter"] // 4 // 8 * 8
     mlp = dict(kind="moe", router=dict(experts=8, top=2), expert=dict(ff=ff), shared=dict(ff=ff))
-    kinds = [dict(type="mlstm", mixer=dict(heads=H, dim=hd, vdim=hd, gate_cap=15.0)),
+    kinds = [dict(type="mlstm", mixer=dict(heads=H, dim=hd, vdim=hd, gate_cap=12.0)),
              dict(type="latent_attention", mixer=dict(heads=H, dim=hd, rot_dim=64, vdim=hd, kv_rank=512, scale=(hd + 64) ** -0.5,
-                                                      rot=dict(base=500000.0, dims=64))),
+                                                      rot=dict(base=100000.0, dims=64))),
              dict(type="retention", mixer=dict(heads=H, dim=hd, vdim=hd, decay=[1 - 2.0 ** -(5 + h % 4) for h in range(H)],
-                                               rot=dict(base=1e6, dims=hd)))]
+                                               rot=dict(base=10000.0, dims=hd)))]
     layers = [dict(kinds[i % 3], mlp=mlp) for i in range(s["layers"])]
     return dict(architecture="Garesun", vocab=s["vocab"], width=W, layers=layers, norm=dict(eps=1e-5), embedding=dict(scale=1.0),
                 token_side=dict(dim=64))
