@@ -21,6 +21,7 @@ Per layer (x: stream, h = LayerNorm(x)):
 from __future__ import annotations
 
 import ctypes as C
+import os
 from types import SimpleNamespace
 from typing import Dict, List, Optional, Sequence
 
@@ -94,6 +95,10 @@ class DecodeRows:
 
 class LanguageModel:
     MAX_DECODE_ROWS = 64
+    # steps of up to this many rows run their big projections on the weight-streaming kernels (with the expert skip); wider
+    # steps take the MFMA GEMM (measured: 1 / 2 / 4 / 8 rows 0.86 / 1.05 / 1.25 / 1.34 ms per step at width 1536 with 2, against
+    # 1.39 / 2.11 ms at 4 / 8 rows with 8).  Environment override for measurements.
+    STREAM_ROWS = int(os.environ.get("VLM_GARESUN_STREAM_ROWS", "2"))
     STATEFUL = True                # recurrent layers: a step that ran cannot be taken back by moving the cache offset
     supports_logits_to_keep = True
 
@@ -203,7 +208,7 @@ class LanguageModel:
         M, K = a.shape
         N = w.shape[0]
         want = out.dtype if out is not None else (out_dtype or a.dtype)
-        if (not accumulate and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and want == torch.bfloat16 and M > 8 and K % 8 == 0 and N % 8 == 0
+        if (not accumulate and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and want == torch.bfloat16 and M > self.STREAM_ROWS and K % 8 == 0 and N % 8 == 0
                 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and (out is None or out.stride(0) % 8 == 0)
                 and a.data_ptr() % 16 == 0 and (out is None or out.data_ptr() % 16 == 0)):
             return ops.gemm(a, w, out=out)
@@ -285,7 +290,7 @@ class LanguageModel:
         tok_seq_d, tok_pos_d, cu_d, slot_d, pos0_d, ids_d = pl.tok_seq, pl.tok_pos, pl.cu, pl.slot, pl.pos0, pl.ids
         pool, bt = self.pool, self.pool.block_table
         is32 = T == f32
-        few = Tn <= 8 and not is32           # decode rows over bf16 weights: weight-streaming projections with the expert skip
+        few = Tn <= self.STREAM_ROWS and not is32           # decode rows over bf16 weights: weight-streaming projections with the expert skip
         x = ops.embed_scale_f32(ids_d, self._w["embed"], cfg.embedding_scale)
         keep = [pl.md, ids_d]
         for i, ns in enumerate(self._L):
@@ -349,7 +354,7 @@ class LanguageModel:
                 keep += [qabs, ol]
             if gate is not None:
                 ops.moe_relu2_gate(col("up"), gate, ns.E, ns.ff, ns.sff, cat[:, ns.koff["ff"]:])
-            if T == torch.bfloat16 and Tn > 8:
+            if T == torch.bfloat16 and Tn > self.STREAM_ROWS:
                 y = self._linear(cat, ns.wout)
                 ops.stream_add_(x, y)
                 keep.append(y)
