@@ -444,3 +444,19 @@ def test_latent_attention_prompt_form_equals_row_form(dtype):
         w = torch.softmax(torch.einsum("hd,jd->hj", q[t].double(), rows) * 0.3, -1)
         want[t] = torch.einsum("hj,jr->hr", w, rows[:, :R]) * torch.sigmoid(gate[t].double())[:, None]
     assert (a.double() - want).abs().max() < 2e-5 and (b.double() - want).abs().max() < 2e-5
+
+
+def test_sampled_generation_uses_the_device_sampler_and_refuses_what_is_not_built(tmp_path):
+    from mlx_vlm_amd.generate import generate_step
+
+    cfg = H.config(H.MIXED[:3])
+    model = _load(tmp_path, cfg, H.weights(cfg, seed=91), "bfloat16", tokens=1024, seqs=4)
+    p = _ids(20, cfg["vocab"], 5)
+    runs = [[t for t, _ in generate_step(p[None], model, None, None, max_tokens=16, temperature=0.8, top_p=0.9, seed=7)] for _ in range(2)]
+    assert runs[0] == runs[1] and len(runs[0]) == 16 and all(0 <= t < cfg["vocab"] for t in runs[0])
+    other = [t for t, _ in generate_step(p[None], model, None, None, max_tokens=16, temperature=0.8, top_p=0.9, seed=8)]
+    greedy = [t for t, _ in generate_step(p[None], model, None, None, max_tokens=16, temperature=0.0)]
+    assert other != runs[0] or greedy != runs[0]                    # the draw depends on the seed / temperature
+    with pytest.raises(NotImplementedError):
+        list(generate_step(p[None], model, None, None, max_tokens=4, repetition_penalty=1.3))
+    assert len(model.language_model.pool._free_seqs) == 4           # every generation gave its slot back
