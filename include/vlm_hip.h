@@ -630,6 +630,79 @@ int vlm_moe_route(const void* logits, int T, int E, int top, void* gate, void* i
 int vlm_moe_relu2_gate(const void* up, long ldu, const void* gate, int E, int ff, int shared, void* out, long ldo, int rows, int dtype,
                        void* stream);
 
+/* csrc/stream_f32.hip, second part: sublayers that read the stream un-normed and norm their RESULT */
+int vlm_stream_cast(const void* x, void* h, int rows, int D, int dtype, void* stream);
+int vlm_rms_rows(const void* x, const void* w, void* out, int rows, int D, long ldo, float eps, int dtype, void* stream);
+/* y = a, or (rms(a) * wa + rms(b) * wb) / 2 when b is given; x += rms(y * sigmoid(gate + gate_bias)) * w (gate may be NULL);
+ * h (may be NULL): T [rows][D], the updated stream rounded for the next reader */
+int vlm_gated_rms_add(void* x, const void* a, long lda, const void* wa, const void* b, long ldb, const void* wb, const void* gate,
+                      long ldg, const void* gate_bias, const void* w, void* h, int rows, int D, float eps, int dtype, void* stream);
+int vlm_relu2_rows(const void* in, long ldi, void* out, long ldo, int rows, int dim, int dtype, void* stream);
+
+/* csrc/delta_rule.hip: delta-rule recurrences (the update reads the old state), state fp32 [slots][H][D][Dv].
+ * Prepare passes write fp32 rows; the scan + finish take them.  Segments as in vlm_linear_recurrence. */
+typedef struct vlm_delta_prep_general_args {
+  const void *r, *k, *v_in, *a;         /* T projections [.][H * D] at ld */
+  long ld;
+  const void* a_bias;                   /* T [H * D] */
+  const void* low;                      /* T [.][R] at ld_low: input of the decay's second map */
+  long ld_low;
+  const void *w2, *w0;                  /* T [H * D][R], T [H * D] */
+  float *q, *kw, *kr, *v, *w, *b;       /* fp32 [ntok][H * D]: read-out key, write key, unit key, value, decay, removal row a * u */
+  int H, D, R;
+} vlm_delta_prep_general_args;
+int vlm_delta_prep_general(const vlm_delta_prep_general_args* a, int ntok, int dtype, void* stream);
+
+typedef struct vlm_delta_prep_gated_args {
+  const void *q_in, *k_in, *v_in;       /* T projections: q, k [.][KH * D], v [.][H * Dv], all at ld */
+  const void *b_in, *a_in;              /* T [.][H] at ld: write strength and step size pre-activations */
+  long ld;
+  const void *q_conv, *k_conv, *v_conv; /* T [channels][taps], the current token's tap last */
+  const void *A_log, *dt_bias;          /* T [H] */
+  float* conv_state;                    /* fp32 [slots][taps - 1][2 KH D + H Dv]: the last inputs before the segment (q | k | v) */
+  const int *seg_start, *seg_slot, *seg_pos0;
+  float *q, *k, *v, *beta, *g;          /* fp32 out: q, k [ntok][KH * D] (unit vectors, q times qscale), v [ntok][H * Dv], [ntok][H] */
+  float qscale;
+  int H, KH, D, Dv, taps;
+} vlm_delta_prep_gated_args;
+/* also moves the slots' convolution inputs to the end of the segments (after every token has read them) */
+int vlm_delta_prep_gated(const vlm_delta_prep_gated_args* a, int nseg, int ntok, int dtype, void* stream);
+
+typedef struct vlm_delta_rule_args {
+  int mode;                             /* 0 = gated: S' = g S, u = beta (v - S'^T k), S = S' + k u^T; 1 = general: S = diag(w) S -
+                                           b (kr^T S) + kw v^T with both terms reading the old S.  o = S^T q. */
+  const float *q, *kw, *kr;             /* fp32 rows at ldk, head h reads key head h / (H / KH) at + kh * D (kr: mode 1 only) */
+  const float* v;                       /* fp32 rows at ldv, head h at + h * Dv */
+  long ldk, ldv;
+  const float *w, *b;                   /* mode 1: fp32 rows at ldk */
+  const float *beta, *g;                /* mode 0: fp32 [ntok][H] */
+  const int *seg_start, *seg_slot, *seg_pos0;
+  float* state;                         /* [slots][H][D][Dv] */
+  float* raw;                           /* scratch fp32 [ntok][H][Dv] */
+  const void* gate;                     /* T rows at ldg: output gate pre-activation [H * Dv] */
+  long ldg;
+  const void* normw;                    /* T [H * Dv] or NULL */
+  int gate_act;                         /* 0 = silu, 1 = sigmoid */
+  float eps;
+  void* out;                            /* T rows at ldo */
+  long ldo;
+  int H, KH, D, Dv;
+} vlm_delta_rule_args;
+int vlm_delta_rule(const vlm_delta_rule_args* a, int nseg, int ntok, int dtype, void* stream);
+
+/* csrc/window_attn.hip: grouped-head softmax attention with a sliding window over paged caches: keys fp32 [pages][64][KH * D]
+ * (normed, rotated), values T [pages][64][KH * Dv].  window <= 0: causal without a window.  temp: T [H] or NULL. */
+int vlm_headnorm_rope_rows(const void* x, long ldx, int heads, int D, const void* w, float eps, int rot_dims, const void* inv_freq,
+                           const void* tok_pos, const void* tok_seq, const void* block_table, int max_pages, void* out, void* raw_pool,
+                           int rows, int dtype, void* stream);
+int vlm_window_attn_blocks(const void* q, const void* kpool, const void* vpool, const void* qb_start, const void* qb_count, int nblocks,
+                           const void* tok_seq, const void* tok_pos, const void* block_table, int max_pages, int H, int KH, int D, int Dv,
+                           float scale, const void* temp, int window, const void* gate, long ldgate, void* out, long ldo, int dtype,
+                           void* stream);
+int vlm_window_attn_rows(const void* q, const void* kpool, const void* vpool, const void* tok_seq, const void* tok_pos,
+                         const void* block_table, int max_pages, int H, int KH, int D, int Dv, float scale, const void* temp, int window,
+                         const void* gate, long ldgate, void* out, long ldo, int rows, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -103,6 +103,29 @@ class RecurrenceArgs(C.Structure):
                    ("Dv", c_int), ("gated", c_int)])
 
 
+class DeltaPrepGeneralArgs(C.Structure):
+    """vlm_delta_prep_general_args (include/vlm_hip.h)"""
+    _fields_ = ([(n, c_void_p) for n in ("r", "k", "v_in", "a")] + [("ld", C.c_long), ("a_bias", c_void_p), ("low", c_void_p),
+                ("ld_low", C.c_long), ("w2", c_void_p), ("w0", c_void_p)] + [(n, c_void_p) for n in ("q", "kw", "kr", "v", "w", "b")]
+                + [("H", c_int), ("D", c_int), ("R", c_int)])
+
+
+class DeltaPrepGatedArgs(C.Structure):
+    """vlm_delta_prep_gated_args (include/vlm_hip.h)"""
+    _fields_ = ([(n, c_void_p) for n in ("q_in", "k_in", "v_in", "b_in", "a_in")] + [("ld", C.c_long)]
+                + [(n, c_void_p) for n in ("q_conv", "k_conv", "v_conv", "A_log", "dt_bias", "conv_state", "seg_start", "seg_slot",
+                                           "seg_pos0", "q", "k", "v", "beta", "g")]
+                + [("qscale", c_float), ("H", c_int), ("KH", c_int), ("D", c_int), ("Dv", c_int), ("taps", c_int)])
+
+
+class DeltaRuleArgs(C.Structure):
+    """vlm_delta_rule_args (include/vlm_hip.h)"""
+    _fields_ = ([("mode", c_int)] + [(n, c_void_p) for n in ("q", "kw", "kr", "v")] + [("ldk", C.c_long), ("ldv", C.c_long)]
+                + [(n, c_void_p) for n in ("w", "b", "beta", "g", "seg_start", "seg_slot", "seg_pos0", "state", "raw", "gate")]
+                + [("ldg", C.c_long), ("normw", c_void_p), ("gate_act", c_int), ("eps", c_float), ("out", c_void_p), ("ldo", C.c_long),
+                   ("H", c_int), ("KH", c_int), ("D", c_int), ("Dv", c_int)])
+
+
 DECODE_FUSED_TAIL = 1                       # vlm_decode_args.flags
 DECODE_ACT16 = 2                            # `act` holds 16 x intermediate_size elements (tiled hand-over to the down projection)
 TUNE_MFMA_GEMV, TUNE_ATTN_PAGESPLIT, TUNE_GEMV_VARIANT, TUNE_ATTN_MERGE = 6, 7, 8, 9  # vlm_llm_set_tuning keys (include/vlm_hip.h)
@@ -202,6 +225,20 @@ SIGNATURES = {
                                        c_int, c_void_p]),
     "vlm_moe_route": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "vlm_moe_relu2_gate": (c_int, [c_void_p, C.c_long, c_void_p, c_int, c_int, c_int, c_void_p, C.c_long, c_int, c_int, c_void_p]),
+    "vlm_stream_cast": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "vlm_rms_rows": (c_int, [c_void_p] * 3 + [c_int, c_int, C.c_long, c_float, c_int, c_void_p]),
+    "vlm_gated_rms_add": (c_int, [c_void_p, c_void_p, C.c_long, c_void_p, c_void_p, C.c_long, c_void_p, c_void_p, C.c_long, c_void_p,
+                                  c_void_p, c_void_p, c_int, c_int, c_float, c_int, c_void_p]),
+    "vlm_relu2_rows": (c_int, [c_void_p, C.c_long, c_void_p, C.c_long, c_int, c_int, c_int, c_void_p]),
+    "vlm_delta_prep_general": (c_int, [P(DeltaPrepGeneralArgs), c_int, c_int, c_void_p]),
+    "vlm_delta_prep_gated": (c_int, [P(DeltaPrepGatedArgs), c_int, c_int, c_int, c_void_p]),
+    "vlm_delta_rule": (c_int, [P(DeltaRuleArgs), c_int, c_int, c_int, c_void_p]),
+    "vlm_headnorm_rope_rows": (c_int, [c_void_p, C.c_long, c_int, c_int, c_void_p, c_float, c_int] + [c_void_p] * 4 + [c_int, c_void_p,
+                                       c_void_p, c_int, c_int, c_void_p]),
+    "vlm_window_attn_blocks": (c_int, [c_void_p] * 5 + [c_int] + [c_void_p] * 3 + [c_int] * 5 + [c_float, c_void_p, c_int, c_void_p,
+                                       C.c_long, c_void_p, C.c_long, c_int, c_void_p]),
+    "vlm_window_attn_rows": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_float, c_void_p, c_int, c_void_p, C.c_long, c_void_p, C.c_long,
+                                     c_int, c_int, c_void_p]),
 }
 
 _lib = None

@@ -50,8 +50,8 @@ __device__ __forceinline__ uint32_t pack_bf2(float lo, float hi) {
 __device__ __forceinline__ float rbf(float f) { return bf2f(f2bf(f)); }
 
 // Wave-wide reductions on the DPP data path.  __shfl_xor compiles to ds_bpermute_b32 on gfx950 - an LDS-crossbar round
-// trip of ~100 cycles per step, six dependent steps per reduction, on the critical tail of every GEMV launch (found in the
-// .s of gemv_rowwave_kernel).  DPP operands ride inside the VALU instruction (v_add_f32_dpp): quad swaps, row_half_mirror
+// trip of ~100 cycles per step, six dependent steps per reduction, on the critical tail of every GEMV launch.
+// DPP operands ride inside the VALU instruction (v_add_f32_dpp): quad swaps, row_half_mirror
 // and row_mirror leave every 16-lane row with its row sum; row_bcast:15 (rows 1, 3) and row_bcast:31 (rows 2, 3) carry
 // the row sums up so that lane 63 holds the total, which v_readlane_b32 broadcasts through an SGPR.  Result in EVERY lane
 // (as the xor butterfly gave); fp32 summation order differs from the butterfly's.

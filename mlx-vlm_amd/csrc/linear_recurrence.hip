@@ -19,15 +19,9 @@
 // c in registers.  Tokens are staged 4 / 8 / 16 at a time through LDS (q, k rotated and scaled on the way in).
 #include "common.hpp"
 #include "../../include/vlm_hip.h"
+#include "recurrence_finish.hpp"
 
 namespace {
-
-template <typename T> __device__ __forceinline__ float ld_f(const T* p);
-template <> __device__ __forceinline__ float ld_f<float>(const float* p) { return *p; }
-template <> __device__ __forceinline__ float ld_f<bf16_t>(const bf16_t* p) { return bf2f(*p); }
-template <typename T> __device__ __forceinline__ void st_f(T* p, float v);
-template <> __device__ __forceinline__ void st_f<float>(float* p, float v) { *p = v; }
-template <> __device__ __forceinline__ void st_f<bf16_t>(bf16_t* p, float v) { *p = f2bf(v); }
 
 constexpr int DR = 32;       // state rows per lane
 constexpr int CT = 64;       // state columns per workgroup
@@ -190,32 +184,6 @@ __global__ __launch_bounds__(64) void gate_max_kernel(vlm_recurrence_args p, int
   if (lane == 0) *ms = m;
 }
 
-template <typename T, bool GATED>
-__global__ __launch_bounds__(64) void recurrence_finish_kernel(vlm_recurrence_args p) {
-  const long tok = blockIdx.x;
-  const int h = blockIdx.y, lane = threadIdx.x;
-  const int Dv = p.Dv, C = Dv + (GATED ? 1 : 0);
-  const float* o = p.raw + (tok * p.H + h) * C;
-  float inv = 1.f;
-  if (GATED) inv = 1.f / (fmaxf(fabsf(o[Dv]), expf(-p.mtok[tok * p.H + h])) + 1e-6f);
-  float ss = 0.f;
-  for (int c = lane; c < Dv; c += 64) {
-    const float x = o[c] * inv;
-    ss += x * x;
-  }
-#pragma unroll
-  for (int d = 32; d > 0; d >>= 1) ss += __shfl_xor(ss, d);
-  const float r = 1.0f / sqrtf(ss / (float)Dv + p.eps);
-  const T* g = (const T*)p.g + tok * p.ldg + (long)h * Dv;
-  T* out = (T*)p.out + tok * p.ldo + (long)h * Dv;
-  for (int c = lane; c < Dv; c += 64) {
-    float x = o[c] * inv * r;
-    if (p.normw) x *= ld_f((const T*)p.normw + (long)h * Dv + c);
-    const float gv = ld_f(g + c), sg = 1.f / (1.f + expf(-gv));
-    st_f(out + c, x * (p.gate_act == 0 ? gv * sg : sg));
-  }
-}
-
 template <typename T>
 int run(const vlm_recurrence_args& a, int nseg, int ntok, hipStream_t st) {
   const int gated = a.gated;
@@ -236,8 +204,12 @@ int run(const vlm_recurrence_args& a, int nseg, int ntok, hipStream_t st) {
     hipLaunchKernelGGL((linear_recurrence_kernel<T, false>), grid, block, lds(TB), st, a, P, TB);
   }
   VLM_CHECK_LAUNCH();
-  if (gated) hipLaunchKernelGGL((recurrence_finish_kernel<T, true>), dim3(ntok, a.H), dim3(64), 0, st, a);
-  else hipLaunchKernelGGL((recurrence_finish_kernel<T, false>), dim3(ntok, a.H), dim3(64), 0, st, a);
+  if (gated)
+    hipLaunchKernelGGL((recurrence_finish_kernel<T, true>), dim3(ntok, a.H), dim3(64), 0, st, a.raw, a.H, a.Dv, a.mtok, a.eps,
+                       (const T*)a.g, a.ldg, (const T*)a.normw, a.gate_act, (T*)a.out, a.ldo);
+  else
+    hipLaunchKernelGGL((recurrence_finish_kernel<T, false>), dim3(ntok, a.H), dim3(64), 0, st, a.raw, a.H, a.Dv, (const float*)nullptr,
+                       a.eps, (const T*)a.g, a.ldg, (const T*)a.normw, a.gate_act, (T*)a.out, a.ldo);
   VLM_CHECK_LAUNCH();
   return VLM_OK;
 }

@@ -1,0 +1,339 @@
+// Softmax attention over a paged per-token cache with grouped key / value heads, an optional sliding window, per-head
+// RMS norm of q and k, interleaved-pair rotary positions on the first rot_dims dimensions, a per-head multiplier on the scores
+// and an elementwise sigmoid gate on the output:
+//
+//     s_ij = (q_i . k_j) * scale * temp[h]        j visible from i  <=>  0 <= i - j < window  (window <= 0: every j <= i)
+//     o_i  = sum_j softmax_j(s_ij) v_j * sigmoid(gate_i)
+//
+//   vlm_headnorm_rope_rows   x rows [T][heads][D] (T-typed) -> RMS norm per head (weight [D] shared by the heads, may be NULL)
+//                            -> rotation of the pairs (2 i, 2 i + 1), i < rot_dims / 2, by pos * inv_freq[i] -> fp32, either
+//                            dense [T][heads][D] (queries) or into the paged pool [page][64][heads * D] of the token's sequence
+//                            (keys).  raw_pool (T-typed, same paging): the rows as they came, for designs whose values are the
+//                            un-normed, un-rotated keys (or any separately projected value rows).
+//   vlm_window_attn_blocks   prompt form: workgroup = (block of up to 16 consecutive queries of one sequence, head); tiles of 16
+//                            keys at multiples of 16 counted from the sequence's first token go through LDS once per block, and
+//                            every query runs the same per-tile update in the same order whatever block it sits in (a tile with
+//                            no visible key leaves its running maximum, sum and accumulator untouched bit for bit): a token's
+//                            result does not depend on how the prompt was cut or batched.
+//   vlm_window_attn_rows     decode form: workgroup = (token, head), one key per lane, tiles of 256 keys from the window's edge.
+// Keys are cached in fp32 (norm and rotation are not rounded), values in T.  Scores, softmax and the weighted sum are fp32.
+#include "common.hpp"
+#include "../../include/vlm_hip.h"
+#include "recurrence_finish.hpp"
+
+namespace {
+
+constexpr int PAGE = 64;
+constexpr int QB = 16, KT = 16;
+
+// grid (tokens, heads), one wave
+template <typename T>
+__global__ __launch_bounds__(64) void headnorm_rope_kernel(const T* __restrict__ x, long ldx, int D, const T* __restrict__ w, float eps,
+                                                           int rot_dims, const float* __restrict__ inv_freq,
+                                                           const int* __restrict__ tok_pos, const int* __restrict__ tok_seq,
+                                                           const int* __restrict__ block_table, int max_pages,
+                                                           float* __restrict__ out, T* __restrict__ raw_pool) {
+  const long t = blockIdx.x;
+  const int h = blockIdx.y, nh = gridDim.y, lane = threadIdx.x;
+  const T* src = x + t * ldx + (long)h * D;
+  const int pos = tok_pos[t];
+  long row = t;                                          // dense output row, or the token's place in the pool
+  if (block_table) row = (long)block_table[(long)tok_seq[t] * max_pages + pos / PAGE] * PAGE + pos % PAGE;
+  float* dst = out + (row * nh + h) * D;
+  float ss = 0.f;
+  for (int i = lane; i < D; i += 64) {
+    const float v = ld_f(src + i);
+    ss += v * v;
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+  const float r = w ? 1.0f / sqrtf(ss / (float)D + eps) : 1.f;
+  for (int i = lane; i < D / 2 + (D & 1); i += 64) {     // one pair per lane and trip (an odd last dimension passes alone)
+    const int i0 = 2 * i, i1 = 2 * i + 1;
+    float u = ld_f(src + i0) * r * (w ? ld_f(w + i0) : 1.f);
+    float v = i1 < D ? ld_f(src + i1) * r * (w ? ld_f(w + i1) : 1.f) : 0.f;
+    if (i1 < rot_dims) {
+      float sn, cs;
+      sincosf((float)pos * inv_freq[i], &sn, &cs);
+      const float u2 = u * cs - v * sn;
+      v = v * cs + u * sn;
+      u = u2;
+    }
+    dst[i0] = u;
+    if (i1 < D) dst[i1] = v;
+  }
+  if (raw_pool) {
+    T* rd = raw_pool + (row * nh + h) * D;
+    for (int i = lane; i < D; i += 64) rd[i] = src[i];
+  }
+}
+
+// thread (r16, l16): score of (query r16, key l16) of the tile; then value dimensions l16 + 16 i of query r16
+template <typename T, int NACC>
+__global__ __launch_bounds__(256) void window_attn_block_kernel(const float* __restrict__ q, const float* __restrict__ kpool,
+                                                                const T* __restrict__ vpool, const int* __restrict__ qb_start,
+                                                                const int* __restrict__ qb_count, const int* __restrict__ tok_seq,
+                                                                const int* __restrict__ tok_pos, const int* __restrict__ block_table,
+                                                                int max_pages, int H, int KH, int D, int Dv, float scale,
+                                                                const T* __restrict__ temp, int window, const T* __restrict__ gate,
+                                                                long ldgate, T* __restrict__ out, long ldo) {
+  extern __shared__ __align__(16) float smem[];
+  const int DP = (D + 3) & ~3, KP = DP + 4, VP = NACC * 16;
+  float* qs = smem;                         // [QB][DP]
+  float* ks = qs + QB * DP;                 // [KT][KP]
+  float* vs = ks + KT * KP;                 // [KT][VP]
+  float* ps = vs + KT * VP;                 // [QB][KT + 1]
+  float* mrun = ps + QB * (KT + 1);         // [QB]
+  float* lrun = mrun + QB;                  // [QB]
+  float* alph = lrun + QB;                  // [QB]
+  const int t0 = qb_start[blockIdx.x], nq = qb_count[blockIdx.x];
+  const int h = blockIdx.y, kh = h / (H / KH), tid = threadIdx.x;
+  const int* bt = block_table + (long)tok_seq[t0] * max_pages;
+  const int pos0 = tok_pos[t0];             // positions of the block's queries: pos0 .. pos0 + nq - 1
+  const int r16 = tid >> 4, l16 = tid & 15;
+  const float sc = scale * (temp ? ld_f(temp + h) : 1.f);
+  for (int d = l16; d < DP; d += 16) qs[r16 * DP + d] = (r16 < nq && d < D) ? q[((long)(t0 + r16) * H + h) * D + d] : 0.f;
+  if (tid < QB) {
+    mrun[tid] = -INFINITY;
+    lrun[tid] = 0.f;
+  }
+  float acc[NACC];
+#pragma unroll
+  for (int b = 0; b < NACC; ++b) acc[b] = 0.f;
+  const int nkeys = pos0 + nq;
+  const int first = window > 0 ? max(0, pos0 - window + 1) : 0;       // the first query's oldest visible key
+  for (int j0 = (first / KT) * KT; j0 < nkeys; j0 += KT) {
+    __syncthreads();
+    {
+      const int key = j0 + r16;
+      float* kd = ks + r16 * KP;
+      float* vd = vs + r16 * VP;
+      if (key < nkeys) {
+        const long rowk = (long)bt[key / PAGE] * PAGE + key % PAGE;
+        const float* ksrc = kpool + (rowk * KH + kh) * D;
+        const T* vsrc = vpool + (rowk * KH + kh) * Dv;
+        for (int d = l16; d < DP; d += 16) kd[d] = d < D ? ksrc[d] : 0.f;
+        for (int d = l16; d < VP; d += 16) vd[d] = d < Dv ? ld_f(vsrc + d) : 0.f;
+      } else {
+        for (int d = l16; d < DP; d += 16) kd[d] = 0.f;
+        for (int d = l16; d < VP; d += 16) vd[d] = 0.f;
+      }
+    }
+    __syncthreads();
+    {
+      const float4* qr = reinterpret_cast<const float4*>(qs + r16 * DP);
+      const float4* kr = reinterpret_cast<const float4*>(ks + l16 * KP);
+      float d = 0.f;
+      for (int i = 0; i < DP / 4; ++i) {
+        const float4 a = qr[i], b = kr[i];
+        d = fmaf(a.x, b.x, d);
+        d = fmaf(a.y, b.y, d);
+        d = fmaf(a.z, b.z, d);
+        d = fmaf(a.w, b.w, d);
+      }
+      const int dist = pos0 + r16 - (j0 + l16);
+      const bool seen = r16 < nq && dist >= 0 && (window <= 0 || dist < window);
+      ps[r16 * (KT + 1) + l16] = seen ? d * sc : -INFINITY;
+    }
+    __syncthreads();
+    if (tid < QB) {                         // per query: running maximum, tile weights, running sum (fixed order over the tile)
+      float s[KT];
+#pragma unroll
+      for (int k = 0; k < KT; ++k) s[k] = ps[tid * (KT + 1) + k];
+      float mt = s[0];
+#pragma unroll
+      for (int k = 1; k < KT; ++k) mt = fmaxf(mt, s[k]);
+      const float m_old = mrun[tid], m_new = fmaxf(m_old, mt);
+      float sum = 0.f;
+#pragma unroll
+      for (int k = 0; k < KT; ++k) {
+        const float pv = s[k] == -INFINITY ? 0.f : expf(s[k] - m_new);
+        ps[tid * (KT + 1) + k] = pv;
+        sum += pv;
+      }
+      const float al = m_new == -INFINITY || m_old == m_new ? 1.f : expf(m_old - m_new);
+      alph[tid] = al;
+      lrun[tid] = lrun[tid] * al + sum;
+      mrun[tid] = m_new;
+    }
+    __syncthreads();
+    const float al = alph[r16];
+#pragma unroll
+    for (int b = 0; b < NACC; ++b) acc[b] *= al;
+#pragma unroll 4
+    for (int k = 0; k < KT; ++k) {
+      const float pv = ps[r16 * (KT + 1) + k];
+#pragma unroll
+      for (int b = 0; b < NACC; ++b) acc[b] = fmaf(pv, vs[k * VP + l16 + 16 * b], acc[b]);
+    }
+  }
+  __syncthreads();
+  if (r16 < nq) {
+    const long t = t0 + r16;
+    const float inv = 1.f / lrun[r16];
+#pragma unroll
+    for (int b = 0; b < NACC; ++b) {
+      const int c = l16 + 16 * b;
+      if (c < Dv) {
+        float o = acc[b] * inv;
+        if (gate) o *= 1.f / (1.f + expf(-ld_f(gate + t * ldgate + (long)h * Dv + c)));
+        st_f(out + t * ldo + (long)h * Dv + c, o);
+      }
+    }
+  }
+}
+
+// workgroup = (token, head): one key per lane and tile for the scores, one value dimension per lane for the weighted sum
+template <typename T, int NACC>
+__global__ __launch_bounds__(256) void window_attn_row_kernel(const float* __restrict__ q, const float* __restrict__ kpool,
+                                                              const T* __restrict__ vpool, const int* __restrict__ tok_seq,
+                                                              const int* __restrict__ tok_pos, const int* __restrict__ block_table,
+                                                              int max_pages, int H, int KH, int D, int Dv, float scale,
+                                                              const T* __restrict__ temp, int window, const T* __restrict__ gate,
+                                                              long ldgate, T* __restrict__ out, long ldo) {
+  extern __shared__ __align__(16) float smem[];
+  float* qs = smem;              // [D]
+  float* ps = qs + ((D + 3) & ~3);  // [256]
+  float* red = ps + 256;         // [8]
+  const long t = blockIdx.x;
+  const int h = blockIdx.y, kh = h / (H / KH), tid = threadIdx.x;
+  const int pos = tok_pos[t];
+  const int* bt = block_table + (long)tok_seq[t] * max_pages;
+  const float sc = scale * (temp ? ld_f(temp + h) : 1.f);
+  for (int i = tid; i < D; i += 256) qs[i] = q[(t * H + h) * D + i];
+  __syncthreads();
+  float m_run = -INFINITY, l_run = 0.f;
+  float acc[NACC];
+#pragma unroll
+  for (int a = 0; a < NACC; ++a) acc[a] = 0.f;
+  const int nkeys = pos + 1;
+  const int first = window > 0 ? max(0, pos - window + 1) : 0;
+  for (int j0 = first; j0 < nkeys; j0 += 256) {
+    const int j = j0 + tid;
+    float s = -INFINITY;
+    if (j < nkeys) {
+      const float* kr = kpool + (((long)bt[j / PAGE] * PAGE + j % PAGE) * KH + kh) * D;
+      float d = 0.f;
+      for (int i = 0; i < D; ++i) d = fmaf(qs[i], kr[i], d);
+      s = d * sc;
+    }
+    float mx = s;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    if ((tid & 63) == 0) red[tid >> 6] = mx;
+    __syncthreads();
+    const float m_new = fmaxf(m_run, fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])));
+    const float pj = j < nkeys ? expf(s - m_new) : 0.f;
+    ps[tid] = pj;
+    float sum = pj;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+    if ((tid & 63) == 0) red[4 + (tid >> 6)] = sum;
+    __syncthreads();
+    const float alpha = expf(m_run - m_new);           // (first tile: exp(-inf) = 0)
+    l_run = l_run * alpha + ((red[4] + red[5]) + (red[6] + red[7]));
+    m_run = m_new;
+    const int nk = min(256, nkeys - j0);
+#pragma unroll
+    for (int a = 0; a < NACC; ++a) {
+      const int dcol = tid + a * 256;
+      if (dcol < Dv) {
+        float v = acc[a] * alpha;
+        for (int jj = 0; jj < nk; ++jj) {
+          const int key = j0 + jj;
+          v = fmaf(ps[jj], ld_f(vpool + (((long)bt[key / PAGE] * PAGE + key % PAGE) * KH + kh) * Dv + dcol), v);
+        }
+        acc[a] = v;
+      }
+    }
+    __syncthreads();
+  }
+  const float inv = 1.f / l_run;
+#pragma unroll
+  for (int a = 0; a < NACC; ++a) {
+    const int c = tid + a * 256;
+    if (c < Dv) {
+      float o = acc[a] * inv;
+      if (gate) o *= 1.f / (1.f + expf(-ld_f(gate + t * ldgate + (long)h * Dv + c)));
+      st_f(out + t * ldo + (long)h * Dv + c, o);
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" int vlm_headnorm_rope_rows(const void* x, long ldx, int heads, int D, const void* w, float eps, int rot_dims,
+                                      const void* inv_freq, const void* tok_pos, const void* tok_seq, const void* block_table,
+                                      int max_pages, void* out, void* raw_pool, int rows, int dtype, void* stream) {
+  if (!x || !tok_pos || !out || heads <= 0 || D <= 0 || rot_dims < 0 || rot_dims > D || (rot_dims & 1) || (rot_dims && !inv_freq) ||
+      ldx < (long)heads * D || rows < 0 || (block_table && (!tok_seq || max_pages <= 0)) || (raw_pool && !block_table))
+    return VLM_ERR_ARG;
+  if (rows == 0) return VLM_OK;
+  if (heads > 65535) return VLM_ERR_SHAPE;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype)
+    hipLaunchKernelGGL(headnorm_rope_kernel<float>, dim3(rows, heads), dim3(64), 0, st, (const float*)x, ldx, D, (const float*)w, eps,
+                       rot_dims, (const float*)inv_freq, (const int*)tok_pos, (const int*)tok_seq, (const int*)block_table, max_pages,
+                       (float*)out, (float*)raw_pool);
+  else
+    hipLaunchKernelGGL(headnorm_rope_kernel<bf16_t>, dim3(rows, heads), dim3(64), 0, st, (const bf16_t*)x, ldx, D, (const bf16_t*)w, eps,
+                       rot_dims, (const float*)inv_freq, (const int*)tok_pos, (const int*)tok_seq, (const int*)block_table, max_pages,
+                       (float*)out, (bf16_t*)raw_pool);
+  VLM_CHECK_LAUNCH();
+  return VLM_OK;
+}
+
+#define WINDOW_ARGS_BAD                                                                                                             \
+  (!q || !kpool || !vpool || !tok_seq || !tok_pos || !block_table || !out || H <= 0 || KH <= 0 || H % KH || D <= 0 || Dv <= 0 ||      \
+   max_pages <= 0 || (gate && ldgate < (long)H * Dv) || ldo < (long)H * Dv)
+
+extern "C" int vlm_window_attn_blocks(const void* q, const void* kpool, const void* vpool, const void* qb_start, const void* qb_count,
+                                      int nblocks, const void* tok_seq, const void* tok_pos, const void* block_table, int max_pages,
+                                      int H, int KH, int D, int Dv, float scale, const void* temp, int window, const void* gate,
+                                      long ldgate, void* out, long ldo, int dtype, void* stream) {
+  if (WINDOW_ARGS_BAD || !qb_start || !qb_count || nblocks < 0) return VLM_ERR_ARG;
+  if (nblocks == 0) return VLM_OK;
+  const int nacc = (Dv + 15) / 16 <= 4 ? 4 : ((Dv + 15) / 16 <= 8 ? 8 : 16);
+  const int DP = (D + 3) & ~3;
+  const size_t lds = ((size_t)QB * DP + (size_t)KT * (DP + 4) + (size_t)KT * nacc * 16 + QB * (KT + 1) + 3 * QB) * sizeof(float);
+  if (Dv > 256 || H > 65535 || lds > 48 * 1024) return VLM_ERR_SHAPE;
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid(nblocks, H);
+#define GO(T, N)                                                                                                                    \
+  hipLaunchKernelGGL((window_attn_block_kernel<T, N>), grid, dim3(256), lds, st, (const float*)q, (const float*)kpool, (const T*)vpool, \
+                     (const int*)qb_start, (const int*)qb_count, (const int*)tok_seq, (const int*)tok_pos, (const int*)block_table,  \
+                     max_pages, H, KH, D, Dv, scale, (const T*)temp, window, (const T*)gate, ldgate, (T*)out, ldo)
+  if (dtype) {
+    if (nacc == 4) GO(float, 4); else if (nacc == 8) GO(float, 8); else GO(float, 16);
+  } else {
+    if (nacc == 4) GO(bf16_t, 4); else if (nacc == 8) GO(bf16_t, 8); else GO(bf16_t, 16);
+  }
+#undef GO
+  VLM_CHECK_LAUNCH();
+  return VLM_OK;
+}
+
+extern "C" int vlm_window_attn_rows(const void* q, const void* kpool, const void* vpool, const void* tok_seq, const void* tok_pos,
+                                    const void* block_table, int max_pages, int H, int KH, int D, int Dv, float scale,
+                                    const void* temp, int window, const void* gate, long ldgate, void* out, long ldo, int rows,
+                                    int dtype, void* stream) {
+  if (WINDOW_ARGS_BAD || rows < 0) return VLM_ERR_ARG;
+  if (rows == 0) return VLM_OK;
+  if (Dv > 1024 || D > 8192 || H > 65535) return VLM_ERR_SHAPE;
+  hipStream_t st = (hipStream_t)stream;
+  const size_t lds = (size_t)(((D + 3) & ~3) + 256 + 8) * sizeof(float);
+  dim3 grid(rows, H);
+#define GO(T, N)                                                                                                                    \
+  hipLaunchKernelGGL((window_attn_row_kernel<T, N>), grid, dim3(256), lds, st, (const float*)q, (const float*)kpool, (const T*)vpool, \
+                     (const int*)tok_seq, (const int*)tok_pos, (const int*)block_table, max_pages, H, KH, D, Dv, scale,              \
+                     (const T*)temp, window, (const T*)gate, ldgate, (T*)out, ldo)
+  const int nacc = (Dv + 255) / 256;
+  if (dtype) {
+    if (nacc == 1) GO(float, 1); else if (nacc == 2) GO(float, 2); else GO(float, 4);
+  } else {
+    if (nacc == 1) GO(bf16_t, 1); else if (nacc == 2) GO(bf16_t, 2); else GO(bf16_t, 4);
+  }
+#undef GO
+  VLM_CHECK_LAUNCH();
+  return VLM_OK;
+}

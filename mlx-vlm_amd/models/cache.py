@@ -643,9 +643,12 @@ def make_prompt_cache(model, max_kv_size: Optional[int] = None):
 # because the recurrence kernels ignore the stored state of a segment that begins at position 0 (nothing is cleared).
 class HybridPool(KVPool):
     def __init__(self, n_layers: int, row_layers, state_layers, max_tokens: int, max_seqs: int, device="cuda",
-                 dtype=torch.bfloat16, max_pages_per_seq: Optional[int] = None):
-        """row_layers: {layer: row width} for layers that write one cached row per token;
-        state_layers: {layer: (heads, rows, cols, has_scalar)}: fp32 state [heads, rows, cols] (+ one fp32 scalar per head)"""
+                 dtype=torch.bfloat16, max_pages_per_seq: Optional[int] = None, aux_layers=None):
+        """row_layers: {key: row width, or (row width, dtype)} for layers that write cached rows per token (key: the layer
+        index, or any sortable key when a layer keeps several row caches, e.g. (layer, "k") / (layer, "v"));
+        state_layers: {layer: (heads, rows, cols, has_scalar)}: fp32 state [heads, rows, cols] (+ one fp32 scalar per head);
+        aux_layers: {layer: shape}: further fp32 state per sequence slot, [max_seqs, *shape] (e.g. the last inputs of a
+        short convolution)"""
         self.n_layers = n_layers
         self.n_kv_heads = self.head_dim = 0                    # (no per-head K / V pages in this pool)
         self.n_pages = (max_tokens + PAGE - 1) // PAGE
@@ -654,7 +657,12 @@ class HybridPool(KVPool):
         self.identity = False
         self.device = device
         self.dtype = dtype
-        self.rows = {int(l): torch.zeros(self.n_pages, PAGE, int(w), dtype=dtype, device=device) for l, w in row_layers.items()}
+        self.rows = {}
+        for l, w in row_layers.items():
+            w, dt = (w if isinstance(w, tuple) else (w, dtype))
+            self.rows[int(l) if not isinstance(l, tuple) else l] = torch.zeros(self.n_pages, PAGE, int(w), dtype=dt, device=device)
+        self.aux = {int(l): torch.zeros(max_seqs, *[int(d) for d in shape], dtype=torch.float32, device=device)
+                    for l, shape in (aux_layers or {}).items()}
         self.state = {int(l): torch.zeros(max_seqs, h, r, c, dtype=torch.float32, device=device)
                       for l, (h, r, c, _) in state_layers.items()}
         self.scalar = {int(l): torch.zeros(max_seqs, h, dtype=torch.float32, device=device)
@@ -668,7 +676,7 @@ class HybridPool(KVPool):
 
     @property
     def nbytes(self):
-        return sum(t.numel() * t.element_size() for d in (self.rows, self.state, self.scalar) for t in d.values())
+        return sum(t.numel() * t.element_size() for d in (self.rows, self.state, self.scalar, self.aux) for t in d.values())
 
     @property
     def free_pages(self) -> int:
@@ -745,6 +753,8 @@ class RecurrentCache:
         out = [pool.state[self._layer][s]]
         if self._layer in pool.scalar:
             out.append(pool.scalar[self._layer][s])
+        if self._layer in pool.aux:
+            out.append(pool.aux[self._layer][s])
         return out
 
     @property

@@ -700,3 +700,95 @@ def moe_relu2_gate(up, gate, E, ff, shared, out):
     check(_lib.lib().vlm_moe_relu2_gate(_p(up), up.stride(0), _p(gate), int(E), int(ff), int(shared), _p(out), out.stride(0),
                                         up.shape[0], _f32(up), _stream()), "moe_relu2_gate")
     return out
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# Sublayers that read the fp32 stream un-normed and norm / gate their result; delta-rule recurrences; windowed attention.
+def stream_cast(x, dtype, out=None):
+    """fp32 stream x [T, D] -> the serving dtype (one rounding)"""
+    _dev(x, out)
+    if out is None:
+        out = torch.empty(x.shape, dtype=dtype, device=x.device)
+    check(_lib.lib().vlm_stream_cast(_p(x), _p(out), x.shape[0], x.shape[1], _f32(out), _stream()), "stream_cast")
+    return out
+
+
+def rms_rows(x, w, eps, out=None):
+    """RMS norm (weight, no mean) over the fp32 stream x [T, D] -> w's dtype"""
+    _dev(x, w, out)
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise _lib.VlmHipError("rms_rows: contiguous fp32 stream expected")
+    if out is None:
+        out = torch.empty(x.shape, dtype=w.dtype, device=x.device)
+    check(_lib.lib().vlm_rms_rows(_p(x), _p(w), _p(out), x.shape[0], x.shape[1], out.stride(0), float(eps), _f32(w), _stream()),
+          "rms_rows")
+    return out
+
+
+def gated_rms_add_(x, a, w, eps, gate=None, gate_bias=None, b=None, wa=None, wb=None, h=None):
+    """x += rms(y * sigmoid(gate + gate_bias)) * w with y = a, or (rms(a) wa + rms(b) wb) / 2 for two branches; h (same shape
+    as x, serving dtype) receives the rounded updated stream"""
+    _dev(x, a, w, gate, gate_bias, b, wa, wb, h)
+    if x.dtype != torch.float32 or not x.is_contiguous() or (h is not None and not h.is_contiguous()):
+        raise _lib.VlmHipError("gated_rms_add: contiguous fp32 stream expected")
+    check(_lib.lib().vlm_gated_rms_add(_p(x), _p(a), a.stride(0), _p(wa), _p(b), b.stride(0) if b is not None else 0, _p(wb), _p(gate),
+                                       gate.stride(0) if gate is not None else 0, _p(gate_bias), _p(w), _p(h), x.shape[0], x.shape[1],
+                                       float(eps), _f32(a), _stream()), "gated_rms_add")
+    return x
+
+
+def relu2_rows(up, out=None):
+    """out = max(up, 0)^2 (2-D views with a row pitch)"""
+    _dev(up, out)
+    if out is None:
+        out = torch.empty(up.shape, dtype=up.dtype, device=up.device)
+    check(_lib.lib().vlm_relu2_rows(_p(up), up.stride(0), _p(out), out.stride(0), up.shape[0], up.shape[1], _f32(up), _stream()),
+          "relu2_rows")
+    return out
+
+
+def delta_prep_general(args: "_lib.DeltaPrepGeneralArgs", ntok: int, dtype_f32: bool):
+    check(_lib.lib().vlm_delta_prep_general(C.byref(args), int(ntok), int(bool(dtype_f32)), _stream()), "delta_prep_general")
+
+
+def delta_prep_gated(args: "_lib.DeltaPrepGatedArgs", nseg: int, ntok: int, dtype_f32: bool):
+    check(_lib.lib().vlm_delta_prep_gated(C.byref(args), int(nseg), int(ntok), int(bool(dtype_f32)), _stream()), "delta_prep_gated")
+
+
+def delta_rule(args: "_lib.DeltaRuleArgs", nseg: int, ntok: int, dtype_f32: bool):
+    check(_lib.lib().vlm_delta_rule(C.byref(args), int(nseg), int(ntok), int(bool(dtype_f32)), _stream()), "delta_rule")
+
+
+def headnorm_rope_rows(x, heads, D, w, eps, rot_dims, inv_freq, tok_pos, out, tok_seq=None, block_table=None, raw_pool=None):
+    """x: 2-D view at the first head's column (row pitch = stride(0)).  Per head: RMS norm with w [D] (None: no norm), pair
+    rotation of the first rot_dims dimensions -> fp32 `out`: dense [T, heads * D], or (with block_table) the paged pool
+    [pages, 64, heads * D]; raw_pool: the un-normed rows in x's dtype, same paging"""
+    _dev(x, w, inv_freq, tok_pos, out, tok_seq, block_table, raw_pool)
+    if out.dtype != torch.float32:
+        raise _lib.VlmHipError("headnorm_rope_rows: fp32 output expected")
+    check(_lib.lib().vlm_headnorm_rope_rows(_p(x), x.stride(0), int(heads), int(D), _p(w), float(eps), int(rot_dims), _p(inv_freq),
+                                            _p(tok_pos), _p(tok_seq), _p(block_table),
+                                            block_table.shape[1] if block_table is not None else 0, _p(out), _p(raw_pool), x.shape[0],
+                                            _f32(x), _stream()), "headnorm_rope_rows")
+    return out
+
+
+def window_attn_blocks(q, kpool, vpool, qb_start, qb_count, tok_seq, tok_pos, block_table, H, KH, D, Dv, scale, out, temp=None, window=0,
+                       gate=None):
+    """prompt form of the windowed attention: q fp32 [T, H * D]; out / gate: 2-D views [T, H * Dv] in vpool's dtype"""
+    _dev(q, kpool, vpool, qb_start, qb_count, tok_seq, tok_pos, block_table, out, temp, gate)
+    check(_lib.lib().vlm_window_attn_blocks(_p(q), _p(kpool), _p(vpool), _p(qb_start), _p(qb_count), qb_start.numel(), _p(tok_seq),
+                                            _p(tok_pos), _p(block_table), block_table.shape[1], int(H), int(KH), int(D), int(Dv),
+                                            float(scale), _p(temp), int(window), _p(gate), gate.stride(0) if gate is not None else 0,
+                                            _p(out), out.stride(0), _f32(vpool), _stream()), "window_attn_blocks")
+    return out
+
+
+def window_attn_rows(q, kpool, vpool, tok_seq, tok_pos, block_table, H, KH, D, Dv, scale, out, temp=None, window=0, gate=None):
+    """decode form of the windowed attention (one workgroup per token and head)"""
+    _dev(q, kpool, vpool, tok_seq, tok_pos, block_table, out, temp, gate)
+    check(_lib.lib().vlm_window_attn_rows(_p(q), _p(kpool), _p(vpool), _p(tok_seq), _p(tok_pos), _p(block_table), block_table.shape[1],
+                                          int(H), int(KH), int(D), int(Dv), float(scale), _p(temp), int(window), _p(gate),
+                                          gate.stride(0) if gate is not None else 0, _p(out), out.stride(0), q.shape[0], _f32(vpool),
+                                          _stream()), "window_attn_rows")
+    return out
