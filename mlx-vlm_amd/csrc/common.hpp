@@ -81,8 +81,7 @@ __device__ __forceinline__ float wave_max(float v) {
 // lane l <-> lane l ^ 16 / l ^ 32 exchanges as ONE gfx950 instruction each (v_permlane16_swap_b32 / v_permlane32_swap_b32:
 // with both operands = v, the results are [r0 r0 r2 r2] | [r1 r1 r3 r3] resp. [lo lo] | [hi hi]) instead of a ds_bpermute.
 // COMPILER TRAP (hipcc / ROCm 7.2; the one gemv_bf16.hip documents): __builtin_bit_cast applied to a vector ELEMENT
-// (r[1]) silently reads element 0 - found in the .s as `v_add_f32 v2, v66, v66` after the swap, and on the GPU as wrong
-// attention.  The elements are copied to scalars first.
+// (r[1]) silently reads element 0 (seen on the GPU as wrong attention).  The elements are copied to scalars first.
 __device__ __forceinline__ void vlm_xor16_pair(float v, float& a, float& b) {
   typedef unsigned int u32x2_t_ __attribute__((ext_vector_type(2)));
   const u32x2_t_ r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned, v), __builtin_bit_cast(unsigned, v), false, false);

@@ -16,16 +16,15 @@
 // the sequence's slot - or is zero when the segment starts at position 0, so a slot that is used again needs no clearing -
 // and goes back there.
 //
-// Scan work split: workgroup = (segment, head, tile of 64 state columns), P parts of 64 lanes; lane c of part p holds rows
-// [DR p, DR p + DR) of column c in registers.  D <= 128 runs with P = 1 (one wave, no barrier inside the token loop); larger
-// heads add the parts' partial sums of S^T k through LDS, one barrier per token.
+// Scan work split: workgroup = (segment, head, tile of 32 state columns) = four waves of 8 columns; eight neighbouring lanes
+// hold the eight parts of one state column's rows in registers (heads up to 1024 wide).
 #include "common.hpp"
 #include "../../include/vlm_hip.h"
 #include "recurrence_finish.hpp"
 
 namespace {
 
-constexpr int CT = 64;       // state columns per workgroup
+constexpr int CT = 32;       // state columns per workgroup (four waves of eight)
 
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.f / (1.f + expf(-x)); }
 __device__ __forceinline__ float softplus_f(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
@@ -152,23 +151,35 @@ __global__ __launch_bounds__(256) void delta_conv_state_kernel(vlm_delta_prep_ga
 }
 
 // ------------------------------------------------------------------------------------------------------------------- scan
+// lane = (column c = lane >> 3 of the wave's 8, row group rg = lane & 7): rows [DR rg, DR rg + DR) of one state column in
+// registers; the eight lanes of a column are half a DPP row, so S^T k and S^T q are DR fused multiply-adds per lane and three
+// DPP exchanges - no barrier and no LDS traffic inside the token loop besides the broadcast reads of the token's vectors.
+constexpr int RG = 8;        // lanes (row groups) per state column
+constexpr int CW = 64 / RG;  // columns per wave
+__device__ __forceinline__ float group_sum(float v) {
+  v += vlm_dpp<0xB1, 0xf>(0.f, v);     // quad_perm [1,0,3,2]
+  v += vlm_dpp<0x4E, 0xf>(0.f, v);     // quad_perm [2,3,0,1]
+  v += vlm_dpp<0x141, 0xf>(0.f, v);    // row_half_mirror: the other quad of the eight lanes
+  return v;
+}
+
 template <int DR, bool GENERAL>
-__global__ __launch_bounds__(512) void delta_scan_kernel(vlm_delta_rule_args p, int P, int TB) {
+__global__ __launch_bounds__(256) void delta_scan_kernel(vlm_delta_rule_args p, int TB) {
   extern __shared__ __align__(16) float smem[];
+  constexpr int GP = DR + 4;              // a row group's pitch in LDS (the four groups' reads of one instruction spread over the banks)
+  constexpr int DP = RG * GP, NV = GENERAL ? 5 : 2;
   const int seg = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * CT;
-  const int D = p.D, Dv = p.Dv, DP = P * DR;
-  const int tid = threadIdx.x, nthr = blockDim.x;
-  const int part = tid / CT, lane = tid % CT, col = c0 + lane, row0 = part * DR;
+  const int D = p.D, Dv = p.Dv;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int rg = lane & (RG - 1), cl = wave * CW + lane / RG, col = c0 + cl, row0 = rg * DR;
   const int kh = h / (p.H / p.KH);
   float* ks = smem;                       // [TB][DP] write key
-  float* us = ks + TB * DP;               // [TB][DP] read key (GENERAL; the gated form reads with the write key)
-  float* qs = us + (GENERAL ? TB * DP : 0);      // [TB][DP]
-  float* ws = qs + TB * DP;               // [TB][DP] decay per key channel (GENERAL)
+  float* qs = ks + TB * DP;               // [TB][DP] read-out key
+  float* us = qs + TB * DP;               // [TB][DP] read key   (GENERAL; the gated form reads with the write key)
+  float* ws = us + (GENERAL ? TB * DP : 0);      // [TB][DP] decay per key channel (GENERAL)
   float* bs = ws + (GENERAL ? TB * DP : 0);      // [TB][DP] removal row (GENERAL)
-  float* vs = bs + (GENERAL ? TB * DP : 0);      // [TB][CT]
+  float* vs = smem + NV * TB * DP;        // [TB][CT]
   float* sc = vs + TB * CT;               // [TB][2]: g, beta (gated)
-  float* po = sc + TB * 2;                // [TB][P][CT] partial read-outs
-  float* pd = po + TB * P * CT;           // [2][P][CT] partial S^T k of the current token (P > 1)
   const int t_begin = p.seg_start[seg], t_end = p.seg_start[seg + 1];
   const int slot = p.seg_slot[seg], pos0 = p.seg_pos0[seg];
   float* S = p.state + ((long)slot * p.H + h) * (long)D * Dv;
@@ -180,19 +191,21 @@ __global__ __launch_bounds__(512) void delta_scan_kernel(vlm_delta_rule_args p, 
   }
   for (int t0 = t_begin; t0 < t_end; t0 += TB) {
     const int nb = min(TB, t_end - t0);
-    for (int idx = tid; idx < nb * DP; idx += nthr) {
-      const int t = idx / DP, i = idx % DP;
+    __syncthreads();                      // (the previous block's vectors are no longer read)
+    for (int idx = tid; idx < nb * RG * DR; idx += 256) {
+      const int t = idx / (RG * DR), i = idx % (RG * DR);
       const long off = (long)(t0 + t) * p.ldk + (long)kh * D + i;
+      const int dst = t * DP + (i / DR) * GP + i % DR;
       const bool in = i < D;
-      ks[idx] = in ? p.kw[off] : 0.f;
-      qs[idx] = in ? p.q[off] : 0.f;
+      ks[dst] = in ? p.kw[off] : 0.f;
+      qs[dst] = in ? p.q[off] : 0.f;
       if (GENERAL) {
-        us[idx] = in ? p.kr[off] : 0.f;
-        ws[idx] = in ? p.w[off] : 0.f;
-        bs[idx] = in ? p.b[off] : 0.f;
+        us[dst] = in ? p.kr[off] : 0.f;
+        ws[dst] = in ? p.w[off] : 0.f;
+        bs[dst] = in ? p.b[off] : 0.f;
       }
     }
-    for (int idx = tid; idx < nb * CT; idx += nthr) {
+    for (int idx = tid; idx < nb * CT; idx += 256) {
       const int t = idx / CT, c = c0 + idx % CT;
       vs[idx] = c < Dv ? p.v[(long)(t0 + t) * p.ldv + (long)h * Dv + c] : 0.f;
     }
@@ -202,7 +215,7 @@ __global__ __launch_bounds__(512) void delta_scan_kernel(vlm_delta_rule_args p, 
     }
     __syncthreads();
     for (int t = 0; t < nb; ++t) {
-      const float4* kr = reinterpret_cast<const float4*>((GENERAL ? us : ks) + t * DP + row0);
+      const float4* kr = reinterpret_cast<const float4*>((GENERAL ? us : ks) + t * DP + rg * GP);
       float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;        // four chains, fixed order
       if (GENERAL) {
 #pragma unroll
@@ -228,21 +241,14 @@ __global__ __launch_bounds__(512) void delta_scan_kernel(vlm_delta_rule_args p, 
           d3 = fmaf(s[4 * r + 3], kk.w, d3);
         }
       }
-      float d = (d0 + d1) + (d2 + d3);
-      if (P > 1) {                        // (P is uniform over the workgroup: every lane reaches the barrier)
-        float* buf = pd + (t & 1) * P * CT;
-        buf[part * CT + lane] = d;
-        __syncthreads();
-        d = 0.f;
-        for (int pp = 0; pp < P; ++pp) d += buf[pp * CT + lane];
-      }
-      const float4* kwr = reinterpret_cast<const float4*>(ks + t * DP + row0);
-      const float4* qr = reinterpret_cast<const float4*>(qs + t * DP + row0);
-      const float vv = vs[t * CT + lane];
+      const float d = group_sum((d0 + d1) + (d2 + d3));
+      const float4* kwr = reinterpret_cast<const float4*>(ks + t * DP + rg * GP);
+      const float4* qr = reinterpret_cast<const float4*>(qs + t * DP + rg * GP);
+      const float vv = vs[t * CT + cl];
       float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
       if (GENERAL) {
-        const float4* wr = reinterpret_cast<const float4*>(ws + t * DP + row0);
-        const float4* br = reinterpret_cast<const float4*>(bs + t * DP + row0);
+        const float4* wr = reinterpret_cast<const float4*>(ws + t * DP + rg * GP);
+        const float4* br = reinterpret_cast<const float4*>(bs + t * DP + rg * GP);
 #pragma unroll
         for (int r = 0; r < DR / 4; ++r) {
           const float4 kk = kwr[r], qq = qr[r], ww = wr[r], bb = br[r];
@@ -270,18 +276,9 @@ __global__ __launch_bounds__(512) void delta_scan_kernel(vlm_delta_rule_args p, 
           a3 = fmaf(s[4 * r + 3], qq.w, a3);
         }
       }
-      po[(t * P + part) * CT + lane] = (a0 + a1) + (a2 + a3);
+      const float o = group_sum((a0 + a1) + (a2 + a3));
+      if (rg == 0 && col < Dv) p.raw[((long)(t0 + t) * p.H + h) * Dv + col] = o;
     }
-    __syncthreads();
-    for (int idx = tid; idx < nb * CT; idx += nthr) {
-      const int t = idx / CT, cc = idx % CT;
-      if (c0 + cc < Dv) {
-        float o = 0.f;
-        for (int pp = 0; pp < P; ++pp) o += po[(t * P + pp) * CT + cc];
-        p.raw[((long)(t0 + t) * p.H + h) * Dv + c0 + cc] = o;
-      }
-    }
-    __syncthreads();
   }
 #pragma unroll
   for (int r = 0; r < DR; ++r) {
@@ -292,24 +289,26 @@ __global__ __launch_bounds__(512) void delta_scan_kernel(vlm_delta_rule_args p, 
 
 template <int DR, bool GENERAL>
 int launch_scan(const vlm_delta_rule_args& a, int nseg, hipStream_t st) {
-  const int P = (a.D + DR - 1) / DR;
-  if (P * CT > 512) return VLM_ERR_SHAPE;
-  const int DP = P * DR;
-  auto lds = [&](int tb) { return ((size_t)tb * ((GENERAL ? 5 : 2) * DP + CT + 2 + P * CT) + 2 * P * CT) * sizeof(float); };
+  constexpr int DP = RG * (DR + 4), NV = GENERAL ? 5 : 2;
+  auto lds = [&](int tb) { return (size_t)tb * (NV * DP + CT + 2) * sizeof(float); };
   int TB = 16;
-  while (TB > 2 && lds(TB) > 48 * 1024) TB >>= 1;
+  while (TB > 1 && lds(TB) > 48 * 1024) TB >>= 1;
   if (lds(TB) > 48 * 1024) return VLM_ERR_SHAPE;
-  dim3 grid(nseg, a.H, (a.Dv + CT - 1) / CT), block(P * CT);
-  hipLaunchKernelGGL((delta_scan_kernel<DR, GENERAL>), grid, block, lds(TB), st, a, P, TB);
+  dim3 grid(nseg, a.H, (a.Dv + CT - 1) / CT), block(256);
+  hipLaunchKernelGGL((delta_scan_kernel<DR, GENERAL>), grid, block, lds(TB), st, a, TB);
   VLM_CHECK_LAUNCH();
   return VLM_OK;
 }
 
 template <bool GENERAL>
 int run_scan(const vlm_delta_rule_args& a, int nseg, hipStream_t st) {
-  if (a.D <= 32) return launch_scan<32, GENERAL>(a, nseg, st);
-  if (a.D <= 64) return launch_scan<64, GENERAL>(a, nseg, st);
-  return launch_scan<128, GENERAL>(a, nseg, st);
+  if (a.D <= 32) return launch_scan<4, GENERAL>(a, nseg, st);
+  if (a.D <= 64) return launch_scan<8, GENERAL>(a, nseg, st);
+  if (a.D <= 128) return launch_scan<16, GENERAL>(a, nseg, st);
+  if (a.D <= 256) return launch_scan<32, GENERAL>(a, nseg, st);
+  if (a.D <= 512) return launch_scan<64, GENERAL>(a, nseg, st);
+  if (a.D <= 1024) return launch_scan<128, GENERAL>(a, nseg, st);
+  return VLM_ERR_SHAPE;
 }
 
 }  // namespace
