@@ -15,7 +15,8 @@
 //                            every query runs the same per-tile update in the same order whatever block it sits in (a tile with
 //                            no visible key leaves its running maximum, sum and accumulator untouched bit for bit): a token's
 //                            result does not depend on how the prompt was cut or batched.
-//   vlm_window_attn_rows     decode form: workgroup = (token, head), one key per lane, tiles of 256 keys from the window's edge.
+//   vlm_window_attn_rows     decode form: workgroup = (token, head); 16-byte loads of key and value rows when D % 4 == 0 and
+//                            Dv % 8 == 0 (chunks of 1024 keys from the window's edge), else one key per lane in tiles of 256.
 // Keys are cached in fp32 (norm and rotation are not rounded), values in T.  Scores, softmax and the weighted sum are fp32.
 #include "common.hpp"
 #include "../../include/vlm_hip.h"
@@ -260,6 +261,121 @@ __global__ __launch_bounds__(256) void window_attn_row_kernel(const float* __res
   }
 }
 
+__device__ __forceinline__ void load8(const bf16_t* p, float* f) {
+  const uint4 v = *reinterpret_cast<const uint4*>(p);
+  f[0] = bf_lo(v.x); f[1] = bf_hi(v.x); f[2] = bf_lo(v.y); f[3] = bf_hi(v.y);
+  f[4] = bf_lo(v.z); f[5] = bf_hi(v.z); f[6] = bf_lo(v.w); f[7] = bf_hi(v.w);
+}
+__device__ __forceinline__ void load8(const float* p, float* f) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+}
+
+// Decode form for D % 4 == 0 and Dv % 8 == 0: workgroup = (token, head), the window in chunks of KC keys.
+//   scores : thread (key, quarter): the four lanes of a DPP quad read one 64-byte piece of a key row per trip (16-byte loads)
+//            and add their partial dot products; 64 keys per pass, no barrier between passes;
+//   softmax: chunk maximum and sum over the scores in LDS (online across chunks);
+//   values : thread (group of 8 value columns, key part): 16-byte loads of V rows, a wave covers whole rows; the key parts'
+//            partial sums are added through LDS at the end.
+constexpr int KC = 1024;
+template <typename T>
+__global__ __launch_bounds__(256) void window_attn_row_vec_kernel(const float* __restrict__ q, const float* __restrict__ kpool,
+                                                                  const T* __restrict__ vpool, const int* __restrict__ tok_seq,
+                                                                  const int* __restrict__ tok_pos, const int* __restrict__ block_table,
+                                                                  int max_pages, int H, int KH, int D, int Dv, float scale,
+                                                                  const T* __restrict__ temp, int window, const T* __restrict__ gate,
+                                                                  long ldgate, T* __restrict__ out, long ldo) {
+  extern __shared__ __align__(16) float smem[];
+  float* qs = smem;                  // [D]
+  float* sc = qs + D;                // [KC] scores, then weights
+  float* part = sc + KC;             // [256 * 8] partial weighted sums
+  int* rowi = reinterpret_cast<int*>(part + 2048);   // [KC] the chunk's keys as pool rows (page * 64 + place): one table lookup per key
+  __shared__ float red[8];
+  const long t = blockIdx.x;
+  const int h = blockIdx.y, kh = h / (H / KH), tid = threadIdx.x, wave = tid >> 6;
+  const int pos = tok_pos[t];
+  const int* bt = block_table + (long)tok_seq[t] * max_pages;
+  const float scl = scale * (temp ? ld_f(temp + h) : 1.f);
+  for (int i = tid; i < D; i += 256) qs[i] = q[(t * H + h) * D + i];
+  const int ngroups = Dv / 8, nparts = 256 / ngroups;          // value-column groups, key parts
+  const int dg = tid % ngroups, kp = tid / ngroups;
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+  const int nkeys = pos + 1;
+  const int first = window > 0 ? max(0, pos - window + 1) : 0;
+  const int D4 = D / 4;
+  __syncthreads();
+  for (int k0 = first; k0 < nkeys; k0 += KC) {
+    const int nk = min(KC, nkeys - k0);
+    for (int j = tid; j < nk; j += 256) rowi[j] = bt[(k0 + j) / PAGE] * PAGE + (k0 + j) % PAGE;
+    __syncthreads();
+#pragma unroll 2
+    for (int jb = 0; jb < nk; jb += 64) {
+      const int j = jb + (tid >> 2), qp = tid & 3;
+      float d = 0.f;
+      if (j < nk) {
+        const float4* kr = reinterpret_cast<const float4*>(kpool + ((long)rowi[j] * KH + kh) * D);
+        const float4* qr = reinterpret_cast<const float4*>(qs);
+        for (int c = qp; c < D4; c += 4) {
+          const float4 a = qr[c], b = kr[c];
+          d = fmaf(a.x, b.x, d);
+          d = fmaf(a.y, b.y, d);
+          d = fmaf(a.z, b.z, d);
+          d = fmaf(a.w, b.w, d);
+        }
+      }
+      d += vlm_dpp<0xB1, 0xf>(0.f, d);     // quad_perm [1,0,3,2]
+      d += vlm_dpp<0x4E, 0xf>(0.f, d);     // quad_perm [2,3,0,1]
+      if (qp == 0 && j < nk) sc[j] = d * scl;
+    }
+    __syncthreads();
+    float mx = -INFINITY;
+    for (int j = tid; j < nk; j += 256) mx = fmaxf(mx, sc[j]);
+    mx = wave_max(mx);
+    if ((tid & 63) == 0) red[wave] = mx;
+    __syncthreads();
+    const float m_new = fmaxf(m_run, fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])));
+    float sum = 0.f;
+    for (int j = tid; j < nk; j += 256) {
+      const float pj = expf(sc[j] - m_new);
+      sc[j] = pj;
+      sum += pj;
+    }
+    sum = wave_sum(sum);
+    if ((tid & 63) == 0) red[4 + wave] = sum;
+    __syncthreads();
+    const float alpha = expf(m_run - m_new);           // (first chunk: exp(-inf) = 0)
+    l_run = l_run * alpha + ((red[4] + red[5]) + (red[6] + red[7]));
+    m_run = m_new;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] *= alpha;
+    if (kp < nparts) {
+#pragma unroll 4
+      for (int j = kp; j < nk; j += nparts) {
+        float f[8];
+        load8(vpool + ((long)rowi[j] * KH + kh) * Dv + dg * 8, f);
+        const float pj = sc[j];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = fmaf(pj, f[i], acc[i]);
+      }
+    }
+    __syncthreads();                                    // (the next chunk overwrites sc and red)
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) part[tid * 8 + i] = acc[i];
+  __syncthreads();
+  const float inv = 1.f / l_run;
+  for (int c = tid; c < Dv; c += 256) {
+    float o = 0.f;
+    for (int pp = 0; pp < nparts; ++pp) o += part[(pp * ngroups + c / 8) * 8 + (c & 7)];
+    o *= inv;
+    if (gate) o *= 1.f / (1.f + expf(-ld_f(gate + t * ldgate + (long)h * Dv + c)));
+    st_f(out + t * ldo + (long)h * Dv + c, o);
+  }
+}
+
 }  // namespace
 
 extern "C" int vlm_headnorm_rope_rows(const void* x, long ldx, int heads, int D, const void* w, float eps, int rot_dims,
@@ -321,8 +437,21 @@ extern "C" int vlm_window_attn_rows(const void* q, const void* kpool, const void
   if (rows == 0) return VLM_OK;
   if (Dv > 1024 || D > 8192 || H > 65535) return VLM_ERR_SHAPE;
   hipStream_t st = (hipStream_t)stream;
-  const size_t lds = (size_t)(((D + 3) & ~3) + 256 + 8) * sizeof(float);
   dim3 grid(rows, H);
+  if (D % 4 == 0 && Dv % 8 == 0 && Dv <= 2048 && (size_t)(D + 2 * KC + 2048) * sizeof(float) <= 48 * 1024) {
+    const size_t ldsv = (size_t)(D + 2 * KC + 2048) * sizeof(float);
+    if (dtype)
+      hipLaunchKernelGGL(window_attn_row_vec_kernel<float>, grid, dim3(256), ldsv, st, (const float*)q, (const float*)kpool,
+                         (const float*)vpool, (const int*)tok_seq, (const int*)tok_pos, (const int*)block_table, max_pages, H, KH, D, Dv,
+                         scale, (const float*)temp, window, (const float*)gate, ldgate, (float*)out, ldo);
+    else
+      hipLaunchKernelGGL(window_attn_row_vec_kernel<bf16_t>, grid, dim3(256), ldsv, st, (const float*)q, (const float*)kpool,
+                         (const bf16_t*)vpool, (const int*)tok_seq, (const int*)tok_pos, (const int*)block_table, max_pages, H, KH, D,
+                         Dv, scale, (const bf16_t*)temp, window, (const bf16_t*)gate, ldgate, (bf16_t*)out, ldo);
+    VLM_CHECK_LAUNCH();
+    return VLM_OK;
+  }
+  const size_t lds = (size_t)(((D + 3) & ~3) + 256 + 8) * sizeof(float);
 #define GO(T, N)                                                                                                                    \
   hipLaunchKernelGGL((window_attn_row_kernel<T, N>), grid, dim3(256), lds, st, (const float*)q, (const float*)kpool, (const T*)vpool, \
                      (const int*)tok_seq, (const int*)tok_pos, (const int*)block_table, max_pages, H, KH, D, Dv, scale,              \

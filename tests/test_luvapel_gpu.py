@@ -84,36 +84,38 @@ def test_stream_operators_of_the_gated_normed_residual():
         assert (ops.relu2_rows(up.cuda()[:, :30]).float().cpu() - torch.relu(up.float()[:, :30]) ** 2).abs().max() < tol * 10
 
 
+@pytest.mark.parametrize("D", [20, 24])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_window_attention_both_forms_against_a_dense_softmax(dtype):
-    """two sequences at different offsets on scattered pages, query blocks that end inside a key tile, grouped heads, a
-    window shorter and longer than the cached prefix, per-head score multipliers, elementwise output gate"""
+def test_window_attention_both_forms_against_a_dense_softmax(dtype, D):
+    """two sequences at different offsets on scattered pages (one 1890 tokens deep: the decode form walks more than one chunk
+    of keys), query blocks that end inside a key tile, grouped heads, windows shorter and longer than the cached prefix, per-
+    head score multipliers, elementwise output gate.  D = 24 takes the decode form with 16-byte loads, D = 20 the plain one."""
     from mlx_vlm_amd import ops
     from mlx_vlm_amd.models.cache import PAGE
 
-    Hh, G, D = 6, 2, 20
+    Hh, G = 6, 2
     g = torch.Generator().manual_seed(9)
-    bt = torch.zeros(3, 8, dtype=torch.int32)
-    bt[1, :3] = torch.tensor([5, 2, 7])
-    bt[2, :1] = torch.tensor([4])
-    kpool = torch.randn(8, PAGE, G * D, generator=g) * 0.7
-    vpool = torch.randn(8, PAGE, G * D, generator=g).to(dtype)
+    bt = torch.zeros(3, 32, dtype=torch.int32)
+    bt[1, :31] = torch.randperm(31, generator=g).to(torch.int32) + 1
+    bt[2, :1] = 0
+    kpool = torch.randn(32, PAGE, G * D, generator=g) * 0.7
+    vpool = torch.randn(32, PAGE, G * D, generator=g).to(dtype)
     tok_seq = torch.tensor([1] * 37 + [2] * 5, dtype=torch.int32)
-    tok_pos = torch.tensor(list(range(150, 187)) + list(range(5)), dtype=torch.int32)
+    tok_pos = torch.tensor(list(range(1890, 1927)) + list(range(5)), dtype=torch.int32)
     q = torch.randn(42, Hh * D, generator=g)
     gate = torch.randn(42, Hh * D + 8, generator=g).to(dtype)
     temp = (1 + 0.3 * torch.randn(Hh, generator=g)).to(dtype)
     qb_start = torch.tensor([0, 16, 32, 37], dtype=torch.int32).cuda()
     qb_count = torch.tensor([16, 16, 5, 5], dtype=torch.int32).cuda()
-    for window in (0, 1, 3, 16, 17, 40, 64, 65, 500):
+    rows = {sq: (kpool[bt[sq].long()].reshape(-1, G, D).double(), vpool[bt[sq].long()].reshape(-1, G, D).double()) for sq in (1, 2)}
+    for window in (0, 1, 3, 16, 17, 40, 64, 65, 500, 1024, 1025, 1800):
         want = torch.zeros(42, Hh, D, dtype=F64)
         for t in range(42):
             sq, pos = int(tok_seq[t]), int(tok_pos[t])
             lo = max(0, pos - window + 1) if window > 0 else 0
             for h in range(Hh):
                 kh = h // (Hh // G)
-                ks = torch.stack([kpool[bt[sq, j // PAGE], j % PAGE, kh * D:(kh + 1) * D] for j in range(lo, pos + 1)]).double()
-                vs = torch.stack([vpool[bt[sq, j // PAGE], j % PAGE, kh * D:(kh + 1) * D] for j in range(lo, pos + 1)]).double()
+                ks, vs = rows[sq][0][lo:pos + 1, kh], rows[sq][1][lo:pos + 1, kh]
                 w = torch.softmax(ks @ q[t, h * D:(h + 1) * D].double() * 0.3 * temp[h].double(), 0)
                 want[t, h] = (w @ vs) * torch.sigmoid(gate[t, h * D:(h + 1) * D].double())
         args = (tok_seq.cuda(), tok_pos.cuda(), bt.cuda(), Hh, G, D, D, 0.3)
