@@ -61,17 +61,25 @@ class ModelConfig:
     @classmethod
     def from_dict(cls, d: Dict[str, Any]) -> "ModelConfig":
         layers = []
-        for i, L in enumerate(d["layers"]):
+        for L in d["layers"]:
             src = L.get("weights_of")
-            lc = LayerConfig(type=L["type"], mixer=dict(L["mixer"]), mlp=(dict(L["mlp"]) if L.get("mlp") else None),
-                             weights_of=None if src is None else int(src))
-            if src is not None:
-                if not 0 <= int(src) < i or layers[int(src)].weights_of is not None:
-                    raise ValueError(f"layer {i}: weights_of must name an earlier layer that has tensors of its own")
-                o = layers[int(src)]
+            layers.append(LayerConfig(type=L["type"], mixer=dict(L["mixer"]), mlp=(dict(L["mlp"]) if L.get("mlp") else None),
+                                      weights_of=None if src is None else int(src)))
+        for i, lc in enumerate(layers):
+            # the source may stand before or after the layer; a source that itself borrows is followed to the owner
+            j, seen = lc.weights_of, {i}
+            while j is not None:
+                if not 0 <= j < len(layers) or j in seen:
+                    raise ValueError(f"layer {i}: weights_of must lead to a layer that has tensors of its own")
+                seen.add(j)
+                if layers[j].weights_of is None:
+                    break
+                j = layers[j].weights_of
+            if j is not None:
+                o = layers[j]
                 if (o.type, o.mixer, o.mlp) != (lc.type, lc.mixer, lc.mlp):
-                    raise ValueError(f"layer {i}: its entry differs from layer {src}, whose weights it uses")
-            layers.append(lc)
+                    raise ValueError(f"layer {i}: its entry differs from layer {j}, whose weights it uses")
+                lc.weights_of = j
         return cls(vocab=int(d["vocab"]), width=int(d["width"]), layers=layers, norm_eps=float(d["norm"]["eps"]),
                    embedding_scale=float((d.get("embedding") or {}).get("scale", 1.0)), eos_token_id=d.get("eos_token_id"))
 

@@ -50,8 +50,9 @@ class LanguageModel(RaggedLanguageModel):
         self._w = dict(embed=shaped(g("embed"), (cfg.vocab, Wd), "embed"), final_norm=shaped(g("final.norm"), (Wd,), "final.norm"),
                        head=shaped(g("head"), (cfg.vocab, Wd), "head"))
         rows, states, aux = {}, {}, {}
-        self._L = []
-        for i, L in enumerate(cfg.layers):
+        self._L = [None] * len(cfg.layers)
+        # layers with tensors of their own first: a borrowing layer may stand before its source
+        for i, L in sorted(enumerate(cfg.layers), key=lambda e: (e[1].weights_of is not None, e[0])):
             if L.weights_of is not None:
                 ns = SimpleNamespace(**vars(self._L[L.weights_of]))
             else:
@@ -105,7 +106,7 @@ class LanguageModel(RaggedLanguageModel):
                 rows[(i, "v")] = (ns.aG * ns.aD, T)                       # the keys as projected
                 if ns.taps > 1:
                     aux[i] = (ns.taps - 1, 2 * ns.G * ns.D + ns.H * ns.Dv)
-            self._L.append(ns)
+            self._L[i] = ns
         self.pool = HybridPool(len(cfg.layers), rows, states, self._kv_pool_tokens, self._max_seqs, device=dev, dtype=T, aux_layers=aux)
         return self
 

@@ -24,8 +24,11 @@ def test_config_reads_every_size_and_refuses_what_the_design_does_not_have():
     with pytest.raises(ValueError):
         ModelConfig.from_dict(bad)
     L = H.mixed_layers()
-    for layers in ([H.shared(L, 0)],                                              # names itself / nothing earlier
-                   [L[0], L[1], H.shared(L, 1), dict(H.shared(L, 1), weights_of=2)],  # a layer without tensors of its own
+    fwd = ModelConfig.from_dict(H.config([H.shared(L, 1), L[1], dict(H.shared(L, 1), weights_of=0), L[0]]))
+    assert [l.weights_of for l in fwd.layers] == [1, None, 1, None]               # a later source; a borrowing source is followed
+    for layers in ([H.shared(L, 0)],                                              # names itself
+                   [L[0], dict(H.shared(L, 0), weights_of=7)],                                      # no such layer
+                   [dict(H.shared(L, 1), weights_of=1), dict(H.shared(L, 1), weights_of=0)],  # no layer with tensors of its own
                    [L[0], dict(H.shared(L, 1), weights_of=0)],                    # another entry than the layer it names
                    [H.parallel(heads=5, kv_heads=2)], [H.parallel(rheads=5, rkv=2)], [H.parallel(rot_dims=5)],
                    [H.parallel(dim=8, rot_dims=10)], [H.parallel(window=0)], [H.parallel(conv=0)]):
@@ -86,6 +89,11 @@ def test_weights_load_on_the_host_and_wrong_shapes_are_refused():
     with pytest.raises(KeyError):
         LanguageModel(ModelConfig.from_dict(cfg), device="cpu", dtype="float32", kv_pool_tokens=64, max_seqs=1).load_weights(missing)
     assert not any(k.startswith("l4.") for k in W)
+    # a borrowing layer may stand before its source
+    L = H.mixed_layers()
+    cfg2 = H.config([H.shared(L, 1), L[1], L[0]])
+    lm2 = LanguageModel(ModelConfig.from_dict(cfg2), device="cpu", dtype="float32", kv_pool_tokens=64, max_seqs=1).load_weights(H.weights(cfg2))
+    assert lm2._L[0].wproj is lm2._L[1].wproj and lm2._L[0].type == "parallel" and lm2._L[2].type == "general_delta"
 
 
 def test_oracle_is_causal_and_its_edges_sit_where_they_should():
