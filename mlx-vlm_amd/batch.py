@@ -767,6 +767,8 @@ class TraceSession:
         """entries: [(request id, next token ids, wanted indices)] -> fp32 logits on the host [n wanted, vocab] or None"""
         batch, want = [], []
         for rid, tokens, w in entries:
+            if len(tokens) == 0:                 # an entry that brings nothing this step asks for nothing
+                continue
             cache = self._live.get(rid)
             if cache is None:
                 cache = self._live[rid] = self.lm.make_cache()

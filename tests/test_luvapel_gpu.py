@@ -108,7 +108,7 @@ def test_window_attention_both_forms_against_a_dense_softmax(dtype, D):
     qb_start = torch.tensor([0, 16, 32, 37], dtype=torch.int32).cuda()
     qb_count = torch.tensor([16, 16, 5, 5], dtype=torch.int32).cuda()
     rows = {sq: (kpool[bt[sq].long()].reshape(-1, G, D).double(), vpool[bt[sq].long()].reshape(-1, G, D).double()) for sq in (1, 2)}
-    for window in (0, 1, 3, 16, 17, 40, 64, 65, 500, 1024, 1025, 1800):
+    for window in (0, 1, 3, 16, 17, 37, 64, 65, 500, 1024, 1025, 1800):
         want = torch.zeros(42, Hh, D, dtype=F64)
         for t in range(42):
             sq, pos = int(tok_seq[t]), int(tok_pos[t])
