@@ -3,6 +3,7 @@ what the design fixes (activation functions, the 1e-6 of the unit vectors, the e
 rotation) lives in the kernels.  Unknown mixer types / feed-forward kinds and inconsistent sizes are refused at load."""
 from __future__ import annotations
 
+import copy
 from dataclasses import dataclass, field
 from typing import Any, Dict, List, Optional
 
@@ -31,7 +32,10 @@ class LayerConfig:
         else:
             _need(m, ("left", "right"), "parallel mixer")
             a, r = m["left"], m["right"]
-            _need(a, ("heads", "kv_heads", "dim", "vdim", "scale", "rot", "mask"), "parallel.left")
+            _need(a, ("heads", "kv_heads", "dim", "scale"), "parallel.left")
+            a.setdefault("vdim", a["dim"])
+            a.setdefault("rot", {"dims": 0, "base": 10000.0})          # an entry without them: no rotation / no window
+            a.setdefault("mask", {"size": None})
             _need(r, ("heads", "kv_heads", "dim", "vdim", "conv"), "parallel.right")
             if int(a["heads"]) % int(a["kv_heads"]) or int(r["heads"]) % int(r["kv_heads"]):
                 raise ValueError("parallel mixer: heads must be a multiple of kv_heads")
@@ -40,12 +44,24 @@ class LayerConfig:
             dims = int(a["rot"]["dims"])
             if dims % 2 or not 0 <= dims <= int(a["dim"]):
                 raise ValueError(f"parallel.left: rot.dims {dims} for head dim {a['dim']}")
-            if int(a["mask"]["size"]) < 1 or int(r["conv"]) < 1:
+            if (a["mask"]["size"] is not None and int(a["mask"]["size"]) < 1) or int(r["conv"]) < 1:
                 raise ValueError("parallel mixer: mask.size and conv are at least 1")
         if self.mlp is not None:
             if self.mlp.get("kind", "dense") != "dense":
                 raise ValueError(f"Luvapel feed-forward kind {self.mlp.get('kind')!r}: 'dense'")
             _need(self.mlp, ("ff",), "feed-forward")
+
+
+def _shape_sizes(lc: LayerConfig):
+    """the sizes of an entry that decide tensor shapes (a borrowing layer must agree on them with its source; window,
+    rotation, score scale are read from the layer's own entry)"""
+    m = lc.mixer
+    if lc.type == "general_delta":
+        sizes = [int(m["heads"]), int(m["dim"])]
+    else:
+        a, r = m["left"], m["right"]
+        sizes = [int(a[k]) for k in ("heads", "kv_heads", "dim")] + [int(r[k]) for k in ("heads", "kv_heads", "dim", "vdim", "conv")]
+    return sizes + [int(lc.mlp["ff"]) if lc.mlp is not None else 0]
 
 
 @dataclass
@@ -63,7 +79,7 @@ class ModelConfig:
         layers = []
         for L in d["layers"]:
             src = L.get("weights_of")
-            layers.append(LayerConfig(type=L["type"], mixer=dict(L["mixer"]), mlp=(dict(L["mlp"]) if L.get("mlp") else None),
+            layers.append(LayerConfig(type=L["type"], mixer=copy.deepcopy(L["mixer"]), mlp=(dict(L["mlp"]) if L.get("mlp") else None),
                                       weights_of=None if src is None else int(src)))
         for i, lc in enumerate(layers):
             # the source may stand before or after the layer; a source that itself borrows is followed to the owner
@@ -77,8 +93,8 @@ class ModelConfig:
                 j = layers[j].weights_of
             if j is not None:
                 o = layers[j]
-                if (o.type, o.mixer, o.mlp) != (lc.type, lc.mixer, lc.mlp):
-                    raise ValueError(f"layer {i}: its entry differs from layer {j}, whose weights it uses")
+                if o.type != lc.type or _shape_sizes(o) != _shape_sizes(lc):
+                    raise ValueError(f"layer {i}: its sizes differ from layer {j}, whose weights it uses")
                 lc.weights_of = j
         return cls(vocab=int(d["vocab"]), width=int(d["width"]), layers=layers, norm_eps=float(d["norm"]["eps"]),
                    embedding_scale=float((d.get("embedding") or {}).get("scale", 1.0)), eos_token_id=d.get("eos_token_id"))

@@ -55,6 +55,8 @@ class LanguageModel(RaggedLanguageModel):
         for i, L in sorted(enumerate(cfg.layers), key=lambda e: (e[1].weights_of is not None, e[0])):
             if L.weights_of is not None:
                 ns = SimpleNamespace(**vars(self._L[L.weights_of]))
+                if L.type == "parallel":                 # what is no tensor comes from the layer's own entry
+                    self._left_constants(ns, L.mixer["left"])
             else:
                 p, m = f"l{i}.", L.mixer
                 ns = SimpleNamespace(type=L.type, norm1=shaped(g(p + "norm1"), (Wd,), p + "norm1"), rg1b=g(p + "rg1.b"))
@@ -70,9 +72,8 @@ class LanguageModel(RaggedLanguageModel):
                     ns.wo = shaped(g(p + "mix.o"), (Wd, H * D), p + "mix.o")
                 else:
                     a, r = m["left"], m["right"]
-                    ns.aH, ns.aG, ns.aD, ns.scale = int(a["heads"]), int(a["kv_heads"]), int(a["dim"]), float(a["scale"])
-                    ns.window, ns.rot_dims = int(a["mask"]["size"]), int(a["rot"]["dims"])
-                    ns.inv_freq = inv_freq(ns.rot_dims, a["rot"]["base"], dev) if ns.rot_dims else None
+                    ns.aH, ns.aG, ns.aD = int(a["heads"]), int(a["kv_heads"]), int(a["dim"])
+                    self._left_constants(ns, a)
                     ns.H, ns.G, ns.D, ns.Dv, ns.taps = int(r["heads"]), int(r["kv_heads"]), int(r["dim"]), int(r["vdim"]), int(r["conv"])
                     pl, pr = p + "mix.left.", p + "mix.right."
                     parts = [("lq", shaped(g(pl + "q"), (ns.aH * ns.aD, Wd), pl + "q")), ("lk", shaped(g(pl + "k"), (ns.aG * ns.aD, Wd), pl + "k")),
@@ -109,6 +110,11 @@ class LanguageModel(RaggedLanguageModel):
             self._L[i] = ns
         self.pool = HybridPool(len(cfg.layers), rows, states, self._kv_pool_tokens, self._max_seqs, device=dev, dtype=T, aux_layers=aux)
         return self
+
+    def _left_constants(self, ns, a):
+        ns.scale, ns.rot_dims = float(a["scale"]), int(a["rot"]["dims"])
+        ns.window = int(a["mask"]["size"]) if a["mask"]["size"] is not None else 0        # 0: every earlier key is seen
+        ns.inv_freq = inv_freq(ns.rot_dims, a["rot"]["base"], self.device) if ns.rot_dims else None
 
     # ------------------------------------------------------------------ cache
     def make_cache(self):

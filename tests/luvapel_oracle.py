@@ -47,11 +47,12 @@ def window_attention(h, W, p, m, eps):
     q, k = (h @ W[p + "q"].T).view(T, H, D), (h @ W[p + "k"].T).view(T, G, D)
     v = k
     pos = torch.arange(T)
-    qn = rotate_pairs(rms(q, eps) * W[p + "q.norm"], pos, m["rot"]["dims"], m["rot"]["base"])
-    kn = rotate_pairs(rms(k, eps) * W[p + "k.norm"], pos, m["rot"]["dims"], m["rot"]["base"])
+    rot, size = m.get("rot") or {"dims": 0, "base": 1.0}, (m.get("mask") or {}).get("size")      # absent: no rotation, no window
+    qn = rotate_pairs(rms(q, eps) * W[p + "q.norm"], pos, rot["dims"], rot["base"])
+    kn = rotate_pairs(rms(k, eps) * W[p + "k.norm"], pos, rot["dims"], rot["base"])
     out = torch.zeros(T, H, D, dtype=h.dtype)
     for i in range(T):
-        lo = max(0, i - m["mask"]["size"] + 1)
+        lo = max(0, i - size + 1) if size else 0
         for hh in range(H):
             g = hh // (H // G)
             s = (kn[lo:i + 1, g] @ qn[i, hh]) * m["scale"] * W[p + "temp"][hh]

@@ -372,6 +372,28 @@ def test_other_sizes(tmp_path):
         assert _close(_portions(lm, ids, [50, 1, 2]), want, dtype), dtype
 
 
+def test_borrowed_weights_before_their_source_and_with_constants_of_their_own(tmp_path):
+    """a layer that uses a LATER layer's tensors, and borrowing layers whose window, score scale and rotation (which are no
+    tensors) differ from their source's"""
+    src = H.parallel(window=9, rot_dims=16, base=10000.0)
+    early, late = H.shared([src], 0), H.shared([src], 0)
+    early["weights_of"], late["weights_of"] = 1, 1
+    early["mixer"]["left"].update(mask=dict(size=3), scale=0.31, rot=dict(base=50.0, dims=8))
+    del late["mixer"]["left"]["mask"], late["mixer"]["left"]["rot"]                # an entry without them: every earlier key, no rotation
+    cfg = H.config([early, src, H.general(), late], vocab=97, width=48, scale=1.3, eps=2e-5)
+    W = H.weights(cfg, seed=31)
+    assert not any(k.startswith(("l0.", "l3.")) for k in W)
+    ids = _ids(90, cfg["vocab"], 37)
+    want = O.Oracle(cfg, W, F64).forward(ids)
+    same = O.Oracle(H.config([H.shared([src], 0) | dict(weights_of=1), src, H.general(), H.shared([src], 0) | dict(weights_of=1)],
+                             vocab=97, width=48, scale=1.3, eps=2e-5), W, F64).forward(ids)
+    assert H.rel_rms(same, want) > 1e-2                                          # the constants of their own matter
+    for dtype in ("float32", "bfloat16"):
+        lm = _load(tmp_path, cfg, W, dtype, tokens=256, name=dtype).language_model
+        assert _close(_whole(lm, ids), want, dtype), dtype
+        assert _close(_portions(lm, ids, [7, 1, 30, 2]), want, dtype), dtype
+
+
 # ------------------------------------------------------------------------------------------------ generation
 def _greedy_oracle(cfg, W, prompt, n):
     orc, ids, toks, margins = O.Oracle(cfg, W, F64), list(prompt), [], []
